@@ -1,0 +1,140 @@
+/*
+ * hogwild_hip.h — C ABI of the MI355X (gfx950) Hogwild! fragmented-KV attention library.
+ *
+ * This is the boundary a binding for the reference's operator API talks to: plain pointers and sizes,
+ * no torch types, no C++ exceptions.  Every entry point returns 0 on success, a negative hw_status for
+ * an argument / support error detected on the host (before any device work is queued), or a positive
+ * hipError_t value if the HIP runtime reported one.
+ *
+ * Entry point  <->  reference interface it replaces (paths relative to the reference tree):
+ *   hw_fused_attention ..... hogwild_fused            src/binding.cu:324-340 (schema :366-367)
+ *   hw_sdpa ................ hogwild_attention        src/binding.cu:255-267, :39-108 (schema :363-364)
+ *                            + launcher v21::hogwild_attention_gpu, src/kernels/kernel_v21.cuh:951-996
+ *   hw_rope ................ hogwild_rope             src/binding.cu:298-308, :217-253; src/rope.cuh:54-62
+ *   hw_workspace_bytes ..... the launcher's private workspace sizing, src/kernels/kernel_v21.cuh:969-980
+ *   hw_problem ............. struct Shape + the launcher argument list, src/common.h:5-20,
+ *                            src/kernels/kernel_v21.cuh:951-957
+ *   hw_status / hw_status_string ... cudaError_t + CUDA_RETURN_ON_ERROR, src/cuda_check.cuh:6-29
+ */
+#ifndef HOGWILD_HIP_H
+#define HOGWILD_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HW_ABI_VERSION 1
+#define HW_MAX_FRAGMENTS 32
+
+typedef enum hw_status {
+    HW_OK = 0,
+    HW_ERR_NULL = -1,          /* a required pointer is NULL */
+    HW_ERR_DTYPE = -2,         /* dtype is not one of hw_dtype */
+    HW_ERR_SHAPE = -3,         /* a dimension is non-positive or inconsistent (Hq % Hkv, RotE > E, odd RotE, ...) */
+    HW_ERR_UNSUPPORTED = -4,   /* shape is valid but no kernel is instantiated for it (never a silent no-op) */
+    HW_ERR_FRAGMENTS = -5,     /* F < 1 or F > HW_MAX_FRAGMENTS */
+    HW_ERR_WORKSPACE = -6,     /* workspace NULL or smaller than hw_workspace_bytes() */
+    HW_ERR_ALIGN = -7,         /* a device pointer is not 16-byte aligned */
+    HW_ERR_NO_DEVICE = -8      /* no usable HIP device */
+} hw_status;
+
+typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
+
+/*
+ * One decode step of one layer.  W workers x S query tokens, Hq query heads sharing Hkv kv heads,
+ * F KV fragments.  Device pointers unless stated otherwise; all tensors contiguous.
+ *
+ *   out        [W, Hq, S, Ev]      dtype     written
+ *   lse        [W, Hq, S]          fp32      written if not NULL: ln sum_visible exp(scale * q.k); -inf for an empty row
+ *   rq         [F, W, Hq, S, E]    dtype     hw_fused_attention only; written if not NULL (the rotated queries the
+ *                                            reference materialises, src/binding.cu:338)
+ *   q          hw_fused_attention: [W, Hq, S, E] un-rotated;  hw_sdpa: [F, W, Hq, S, E] already rotated
+ *   locations  [F, W, S]           int32     query (w,s) sees key l of fragment f iff l <= locations[f,w,s]
+ *                                            (src/kernels/kernel_v21.cuh:96-98)
+ *   cosines, sines [F, W, S, RotE] fp32      hw_fused_attention only (src/rope.cuh:18-51 index convention)
+ *   k, v       HOST arrays of F device pointers; fragment f is [Hkv, len[f], E] / [Hkv, len[f], Ev]
+ *   len        HOST array of F lengths (the reference reads the same numbers from the tensor sizes, src/binding.cu:91)
+ *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
+ *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
+ *   ev_start / ev_stop   optional hipEvent_t recorded on `stream` immediately before / after the attention
+ *                        kernel (not the merge kernel); pass NULL outside of profiling
+ */
+typedef struct hw_problem {
+    int32_t dtype;
+    int32_t F, W, Hq, Hkv, S, E, Ev, RotE;
+    float scale;
+    void* out;
+    float* lse;
+    void* rq;
+    const void* q;
+    const int32_t* locations;
+    const float* cosines;
+    const float* sines;
+    const void* const* k;
+    const void* const* v;
+    const int32_t* len;
+    void* workspace;
+    size_t workspace_bytes;
+    int32_t splits;
+    void* ev_start;
+    void* ev_stop;
+} hw_problem;
+
+/* How a problem is cut into workgroups; filled by hw_plan_debug (host only, no device needed). */
+typedef struct hw_plan {
+    int32_t rows;             /* W*S*(Hq/Hkv): query rows that share one kv head */
+    int32_t row_blocks;       /* 16-row MFMA blocks per workgroup (1 or 2) */
+    int32_t row_groups;       /* workgroups along the row dimension */
+    int32_t tile_tokens;      /* tokens per wave step */
+    int32_t tiles_per_head;   /* sum_f ceil(len[f] / tile_tokens) */
+    int32_t wgs_per_head;     /* split-K factor */
+    int32_t workgroups;       /* grid size of the attention kernel */
+    int32_t tile_begin[HW_MAX_FRAGMENTS + 1];
+    size_t workspace_bytes;
+} hw_plan;
+
+int hw_version(void);
+const char* hw_status_string(int status);
+
+/* Host-only argument check shared by all entry points (pointer checks cover what `fused` != 0 needs). */
+int hw_validate(const hw_problem* p, int fused);
+
+/* Host-only: the split plan for a device with `num_cus` compute units. */
+int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan);
+
+/* Workspace size for the current device. */
+int hw_workspace_bytes(const hw_problem* p, size_t* bytes);
+
+/* Rotate q per fragment in registers and attend; replaces hogwild_fused. */
+int hw_fused_attention(const hw_problem* p, void* stream);
+
+/* Attend with already-rotated queries [F,W,Hq,S,E]; replaces hogwild_sdpa. */
+int hw_sdpa(const hw_problem* p, void* stream);
+
+/* out[F,W,Hq,S,E] = rope(q[W,Hq,S,E], cos/sin[F,W,S,RotE]); replaces hogwild_rope. */
+int hw_rope(void* out, const void* q, const float* cosines, const float* sines, int dtype,
+            int F, int W, int Hq, int S, int E, int RotE, void* stream);
+
+/* Number of compute units of the current device (0 on failure). */
+int hw_device_cus(void);
+
+/* Small HIP-event helpers so a profiling harness needs no other HIP binding. */
+int hw_event_create(void** ev);
+int hw_event_destroy(void* ev);
+int hw_event_record(void* ev, void* stream);
+int hw_event_synchronize(void* ev);
+int hw_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* Streaming read of `bytes` bytes (multiple of 16) from `src`, xor-reduced into sink[0..255]: the plain
+   bandwidth calibration the attention kernel is compared with. */
+int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
+/* Plain copy kernel of known size, used to scale FETCH_SIZE / WRITE_SIZE counters. */
+int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HOGWILD_HIP_H */

@@ -1,0 +1,271 @@
+"""ctypes view of the C ABI in include/hogwild_hip.h.
+
+The library is required: importing this module without a built libhogwild_hip.so raises, and no entry
+point here has a CPU or eager fallback.  Tensors are torch tensors on the GPU; only their pointers,
+sizes and the current HIP stream cross the boundary.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+from typing import List, Optional, Sequence
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
+
+HW_MAX_FRAGMENTS = 32
+HW_F32, HW_F16, HW_BF16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_BF16}
+
+EXPORTS = [
+    "hw_version", "hw_status_string", "hw_validate", "hw_plan_debug", "hw_workspace_bytes",
+    "hw_fused_attention", "hw_sdpa", "hw_rope", "hw_device_cus",
+    "hw_event_create", "hw_event_destroy", "hw_event_record", "hw_event_synchronize", "hw_event_elapsed_ms",
+    "hw_stream_read", "hw_stream_copy",
+]
+
+
+class HwProblem(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("F", C.c_int32), ("W", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32), ("S", C.c_int32),
+        ("E", C.c_int32), ("Ev", C.c_int32), ("RotE", C.c_int32),
+        ("scale", C.c_float),
+        ("out", C.c_void_p), ("lse", C.c_void_p), ("rq", C.c_void_p),
+        ("q", C.c_void_p), ("locations", C.c_void_p), ("cosines", C.c_void_p), ("sines", C.c_void_p),
+        ("k", C.POINTER(C.c_void_p)), ("v", C.POINTER(C.c_void_p)), ("len", C.POINTER(C.c_int32)),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("splits", C.c_int32),
+        ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p),
+    ]
+
+
+class HwPlan(C.Structure):
+    _fields_ = [
+        ("rows", C.c_int32), ("row_blocks", C.c_int32), ("row_groups", C.c_int32), ("tile_tokens", C.c_int32),
+        ("tiles_per_head", C.c_int32), ("wgs_per_head", C.c_int32), ("workgroups", C.c_int32),
+        ("tile_begin", C.c_int32 * (HW_MAX_FRAGMENTS + 1)),
+        ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class HogwildError(RuntimeError):
+    def __init__(self, status: int, where: str):
+        self.status = status
+        super().__init__(f"{where}: status {status}: {status_string(status)}")
+
+
+def _load() -> C.CDLL:
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m inference_lib_amd.build` "
+            "(there is no fallback path for the Hogwild attention operators)")
+    lib = C.CDLL(LIB_PATH)
+    lib.hw_version.restype = C.c_int
+    lib.hw_status_string.restype = C.c_char_p
+    lib.hw_status_string.argtypes = [C.c_int]
+    lib.hw_validate.argtypes = [C.POINTER(HwProblem), C.c_int]
+    lib.hw_plan_debug.argtypes = [C.POINTER(HwProblem), C.c_int, C.POINTER(HwPlan)]
+    lib.hw_workspace_bytes.argtypes = [C.POINTER(HwProblem), C.POINTER(C.c_size_t)]
+    lib.hw_fused_attention.argtypes = [C.POINTER(HwProblem), C.c_void_p]
+    lib.hw_sdpa.argtypes = [C.POINTER(HwProblem), C.c_void_p]
+    lib.hw_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
+                            C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.hw_event_create.argtypes = [C.POINTER(C.c_void_p)]
+    lib.hw_event_destroy.argtypes = [C.c_void_p]
+    lib.hw_event_record.argtypes = [C.c_void_p, C.c_void_p]
+    lib.hw_event_synchronize.argtypes = [C.c_void_p]
+    lib.hw_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
+    lib.hw_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+    lib.hw_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    return lib
+
+
+lib = _load()
+
+
+def status_string(status: int) -> str:
+    return lib.hw_status_string(int(status)).decode()
+
+
+def check(status: int, where: str) -> None:
+    if status != 0:
+        raise HogwildError(status, where)
+
+
+def _frag3(t: torch.Tensor) -> torch.Tensor:
+    """Fragments come as [Hkv, L, D] or [1, Hkv, L, D] (src/binding.cu:85-94)."""
+    if t.dim() == 4:
+        if t.size(0) != 1:
+            raise ValueError("4-D KV fragment must have a leading dimension of 1")
+        return t[0]
+    if t.dim() != 3:
+        raise ValueError("KV fragment must be [Hkv, L, D] or [1, Hkv, L, D]")
+    return t
+
+
+class Problem:
+    """Owns the ctypes arrays of one hw_problem and keeps the tensors alive."""
+
+    def __init__(self, *, q: torch.Tensor, locations: torch.Tensor, keys: Sequence[torch.Tensor],
+                 values: Sequence[torch.Tensor], scale: float, out: torch.Tensor,
+                 cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
+                 rq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                 prerotated: bool = False, splits: int = 0):
+        keys = [_frag3(k) for k in keys]
+        values = [_frag3(v) for v in values]
+        F = len(keys)
+        if len(values) != F or locations.size(0) != F:
+            raise ValueError("fragment count mismatch between keys, values and locations")
+        if F < 1 or F > HW_MAX_FRAGMENTS:
+            raise HogwildError(-5, "Problem")
+        W, Hq, S, Ev = out.shape
+        E = q.size(-1)
+        Hkv = keys[0].size(0)
+        if out.dtype not in _DTYPE_CODE:
+            raise HogwildError(-2, "Problem")
+        expect_q = (F, W, Hq, S, E) if prerotated else (W, Hq, S, E)
+        if tuple(q.shape) != expect_q:
+            raise ValueError(f"queries have shape {tuple(q.shape)}, expected {expect_q}")
+        if tuple(locations.shape) != (F, W, S) or locations.dtype != torch.int32:
+            raise ValueError("locations must be int32 [F, W, S]")
+        tensors = [out, q, locations] + keys + values
+        for f in range(F):
+            if keys[f].size(0) != Hkv or values[f].size(0) != Hkv or keys[f].size(1) != values[f].size(1) \
+                    or keys[f].size(2) != E or values[f].size(2) != Ev:
+                raise ValueError(f"fragment {f} has inconsistent shape")
+            if keys[f].dtype != out.dtype or values[f].dtype != out.dtype:
+                raise ValueError("KV fragments must have the dtype of the output")
+        if q.dtype != out.dtype:
+            raise ValueError("queries must have the dtype of the output")
+        rot = 0
+        if not prerotated:
+            if cosines is None or sines is None:
+                raise ValueError("the fused operator needs cosines and sines")
+            rot = cosines.size(-1)
+            if tuple(cosines.shape) != (F, W, S, rot) or tuple(sines.shape) != (F, W, S, rot):
+                raise ValueError("cosines / sines must be [F, W, S, RotE]")
+            if cosines.dtype != torch.float32 or sines.dtype != torch.float32:
+                raise ValueError("cosines / sines must be float32")
+            tensors += [cosines, sines]
+        if rq is not None:
+            if tuple(rq.shape) != (F, W, Hq, S, E) or rq.dtype != out.dtype:
+                raise ValueError("rotated-query buffer must be [F, W, Hq, S, E] in the output dtype")
+            tensors.append(rq)
+        if lse is not None:
+            if tuple(lse.shape) != (W, Hq, S) or lse.dtype != torch.float32:
+                raise ValueError("lse must be float32 [W, Hq, S]")
+            tensors.append(lse)
+        for t in tensors:
+            if not t.is_contiguous():
+                raise ValueError("all tensors must be contiguous")
+            if t.device != out.device:
+                raise ValueError("all tensors must live on the output's device")
+        self._keep = tensors
+        self.device = out.device
+        self._k = (C.c_void_p * F)(*[k.data_ptr() for k in keys])
+        self._v = (C.c_void_p * F)(*[v.data_ptr() for v in values])
+        self._len = (C.c_int32 * F)(*[k.size(1) for k in keys])
+        p = HwProblem()
+        p.dtype = _DTYPE_CODE[out.dtype]
+        p.F, p.W, p.Hq, p.Hkv, p.S, p.E, p.Ev, p.RotE = F, W, Hq, Hkv, S, E, Ev, rot
+        p.scale = float(scale)
+        p.out = out.data_ptr()
+        p.lse = lse.data_ptr() if lse is not None else None
+        p.rq = rq.data_ptr() if rq is not None else None
+        p.q = q.data_ptr()
+        p.locations = locations.data_ptr()
+        p.cosines = cosines.data_ptr() if cosines is not None else None
+        p.sines = sines.data_ptr() if sines is not None else None
+        p.k = C.cast(self._k, C.POINTER(C.c_void_p))
+        p.v = C.cast(self._v, C.POINTER(C.c_void_p))
+        p.len = C.cast(self._len, C.POINTER(C.c_int32))
+        p.splits = int(splits)
+        self.p = p
+        self.prerotated = prerotated
+        self._ws = None
+
+    def workspace_bytes(self) -> int:
+        n = C.c_size_t(0)
+        with torch.cuda.device(self.device):
+            check(lib.hw_workspace_bytes(C.byref(self.p), C.byref(n)), "hw_workspace_bytes")
+        return n.value
+
+    def set_workspace(self, ws: Optional[torch.Tensor] = None) -> None:
+        if ws is None:
+            ws = torch.empty(self.workspace_bytes(), dtype=torch.uint8, device=self.device)
+        self._ws = ws
+        self.p.workspace = ws.data_ptr()
+        self.p.workspace_bytes = ws.numel() * ws.element_size()
+
+    def set_events(self, start: Optional[int], stop: Optional[int]) -> None:
+        self.p.ev_start = start
+        self.p.ev_stop = stop
+
+    def run(self) -> None:
+        if self._ws is None:
+            self.set_workspace()
+        with torch.cuda.device(self.device):
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            fn = lib.hw_sdpa if self.prerotated else lib.hw_fused_attention
+            check(fn(C.byref(self.p), C.c_void_p(stream)), fn.__name__)
+
+
+def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num_cus: int, splits: int = 0) -> HwPlan:
+    """Host-only split plan (no GPU needed)."""
+    F = len(lens)
+    arr = (C.c_int32 * max(F, 1))(*lens)
+    p = HwProblem()
+    p.F, p.W, p.S, p.Hq, p.Hkv, p.Ev, p.E = F, W, S, Hq, Hkv, Ev, Ev
+    p.len = C.cast(arr, C.POINTER(C.c_int32))
+    p.splits = splits
+    out = HwPlan()
+    check(lib.hw_plan_debug(C.byref(p), num_cus, C.byref(out)), "hw_plan_debug")
+    return out
+
+
+def rope(q: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    F, W, Hq, S, E = out.shape
+    if tuple(q.shape) != (W, Hq, S, E) or q.dtype != out.dtype:
+        raise ValueError("queries must be [W, Hq, S, E] in the output dtype")
+    rot = cosines.size(-1)
+    if tuple(cosines.shape) != (F, W, S, rot) or tuple(sines.shape) != (F, W, S, rot):
+        raise ValueError("cosines / sines must be [F, W, S, RotE]")
+    if cosines.dtype != torch.float32 or sines.dtype != torch.float32:
+        raise ValueError("cosines / sines must be float32")
+    for t in (q, cosines, sines, out):
+        if not t.is_contiguous():
+            raise ValueError("all tensors must be contiguous")
+    with torch.cuda.device(out.device):
+        stream = torch.cuda.current_stream(out.device).cuda_stream
+        check(lib.hw_rope(out.data_ptr(), q.data_ptr(), cosines.data_ptr(), sines.data_ptr(), _DTYPE_CODE[out.dtype],
+                          F, W, Hq, S, E, rot, C.c_void_p(stream)), "hw_rope")
+    return out
+
+
+class Event:
+    """A HIP event created through the library (for per-kernel timing on the op's own stream)."""
+
+    def __init__(self):
+        h = C.c_void_p()
+        check(lib.hw_event_create(C.byref(h)), "hw_event_create")
+        self.handle = h.value
+
+    def record(self, stream: int) -> None:
+        check(lib.hw_event_record(self.handle, C.c_void_p(stream)), "hw_event_record")
+
+    def synchronize(self) -> None:
+        check(lib.hw_event_synchronize(self.handle), "hw_event_synchronize")
+
+    def elapsed_ms(self, stop: "Event") -> float:
+        ms = C.c_float()
+        check(lib.hw_event_elapsed_ms(self.handle, stop.handle, C.byref(ms)), "hw_event_elapsed_ms")
+        return ms.value
+
+    def __del__(self):
+        try:
+            lib.hw_event_destroy(self.handle)
+        except Exception:
+            pass

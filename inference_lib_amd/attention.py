@@ -1,0 +1,76 @@
+"""Host-side mirror of the reference's operator wrappers (python/hogwild/attention.py:19-35, 70-74)
+for the MI355X HIP library.  Same names, argument order and defaults; every function runs the HIP
+kernels through the C ABI and raises if the library is not built — there is no eager fallback here.
+
+When the torch operator binding (hogatt.abi3.so, namespace `libhogatt`) has been built it is loaded
+and used, so that `torch.ops.libhogatt.hogwild_fused(...)` call sites keep working; otherwise the same
+C entry points are called through ctypes.
+"""
+from __future__ import annotations
+
+import os
+from typing import List, Optional
+
+import torch
+
+from . import _lib
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_TORCH_EXT = os.path.join(_HERE, "hogatt.abi3.so")
+HAVE_TORCH_OPS = False
+if os.path.exists(_TORCH_EXT):
+    torch.ops.load_library(_TORCH_EXT)
+    HAVE_TORCH_OPS = True
+
+
+def hogwild_fused(queries: torch.Tensor, locations: torch.Tensor, keys: List[torch.Tensor], values: List[torch.Tensor],
+                  scale: float, fragment_lengths, cosines: torch.Tensor, sines: torch.Tensor, *, rotated_queries, out,
+                  lse: Optional[torch.Tensor] = None):
+    """rope + attention in one pass (python/hogwild/attention.py:19-23).  `fragment_lengths` is accepted
+    for signature compatibility; the lengths are taken from the fragment tensors, which the reference
+    requires to agree with it (src/kernels/kernel_v21.cuh:116-117).  `lse` (float32 [W,Hq,S]) is an
+    addition: natural-log log-sum-exp of the scaled visible logits."""
+    if HAVE_TORCH_OPS and lse is None:
+        torch.ops.libhogatt.hogwild_fused(out, rotated_queries, scale, locations, queries.contiguous(), fragment_lengths,
+                                          keys, values, cosines, sines)
+        return out
+    if HAVE_TORCH_OPS:
+        torch.ops.libhogatt.hogwild_fused_lse(out, rotated_queries, lse, scale, locations, queries.contiguous(),
+                                              fragment_lengths, keys, values, cosines, sines)
+        return out
+    keys = [k.contiguous() for k in keys]        # the reference op copies non-contiguous fragments too, binding.cu:330-337
+    values = [v.contiguous() for v in values]
+    pr = _lib.Problem(q=queries.contiguous(), locations=locations, keys=keys, values=values, scale=scale, out=out,
+                      cosines=cosines, sines=sines, rq=rotated_queries, lse=lse)
+    pr.run()
+    return out
+
+
+def hogwild_sdpa(queries: torch.Tensor, locations: torch.Tensor, keys: List[torch.Tensor], values: List[torch.Tensor],
+                 scale: float, fragment_lengths=None, out=None, lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention with already-rotated queries [F,W,Hq,S,E] (python/hogwild/attention.py:26-35)."""
+    if out is None:
+        out = torch.empty((queries.size(1), queries.size(2), queries.size(3), values[0].size(-1)), dtype=queries.dtype,
+                          device=queries.device)
+    keys = [k.contiguous() for k in keys]
+    values = [v.contiguous() for v in values]
+    if HAVE_TORCH_OPS and lse is None:
+        if fragment_lengths is None:
+            fragment_lengths = torch.tensor([k.size(-2) for k in keys], dtype=torch.int32, device=queries.device)
+        torch.ops.libhogatt.hogwild_sdpa(out, scale, locations, queries.contiguous(), fragment_lengths, keys, values)
+        return out
+    pr = _lib.Problem(q=queries.contiguous(), locations=locations, keys=keys, values=values, scale=scale, out=out, lse=lse,
+                      prerotated=True)
+    pr.run()
+    return out
+
+
+def hogwild_rope(queries: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out=None):
+    """Per-fragment rotation of the queries (python/hogwild/attention.py:70-74)."""
+    if out is None:
+        out = torch.empty((cosines.size(0), queries.size(0), queries.size(1), queries.size(2), queries.size(3)),
+                          dtype=queries.dtype, device=queries.device)
+    if HAVE_TORCH_OPS:
+        torch.ops.libhogatt.hogwild_rope(out, queries, cosines, sines)
+        return out
+    return _lib.rope(queries, cosines, sines, out)

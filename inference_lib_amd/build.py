@@ -1,0 +1,65 @@
+"""In-tree build of the native pieces for gfx950.
+
+  libhogwild_hip.so ... HIP kernels + the C ABI declared in include/hogwild_hip.h
+  hogatt.abi3.so ...... torch operator binding (namespace libhogatt) on top of the C ABI
+
+Run as `python -m inference_lib_amd.build`.  hipcc cross-compiles for gfx950 without a GPU present.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+import sysconfig
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libhogwild_hip.so")
+TORCH_EXT = os.path.join(HERE, "hogatt.abi3.so")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ARCH = "gfx950"
+# packed fp32 VALU ops are switched off for every device compile of this library
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def _run(cmd):
+    print("+", " ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+
+
+def build_library() -> str:
+    srcs = [os.path.join(CSRC, "hogwild_kernels.hip"), os.path.join(CSRC, "hogwild_capi.hip")]
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
+           "-munsafe-fp-atomics", *DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *srcs]
+    _run(cmd)
+    return LIB
+
+
+def build_torch_binding() -> str:
+    import torch
+    from torch.utils import cpp_extension
+
+    inc = cpp_extension.include_paths()
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include", "-I", sysconfig.get_paths()["include"]]
+    for i in inc:
+        cmd += ["-isystem", i]
+    cmd += [os.path.join(CSRC, "hogatt_binding.cpp"), "-o", TORCH_EXT,
+            "-L", HERE, "-lhogwild_hip", "-L", torch_lib, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+            "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}"]
+    _run(cmd)
+    return TORCH_EXT
+
+
+def build_all(with_torch: bool = True) -> None:
+    build_library()
+    if with_torch:
+        build_torch_binding()
+
+
+if __name__ == "__main__":
+    build_all(with_torch="--no-torch" not in sys.argv)

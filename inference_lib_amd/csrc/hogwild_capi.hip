@@ -1,0 +1,263 @@
+// C ABI of the Hogwild! attention library: argument validation, split planning and launches.
+// Validation and planning are pure host code and run before any HIP call, so they can be tested on a
+// machine without a GPU.  No global mutable state apart from an immutable per-device CU-count cache.
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cmath>
+#include <cstring>
+
+#include "../../include/hogwild_hip.h"
+#include "hogwild_kernels.h"
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<int> g_cus[kMaxDevices];   // 0 = not queried yet
+
+int device_cus(int* cus) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HW_ERR_NO_DEVICE;
+    int c = g_cus[dev].load(std::memory_order_relaxed);
+    if (c == 0) {
+        e = hipDeviceGetAttribute(&c, hipDeviceAttributeMultiprocessorCount, dev);
+        if (e != hipSuccess) return (int)e;
+        if (c <= 0) return HW_ERR_NO_DEVICE;
+        g_cus[dev].store(c, std::memory_order_relaxed);
+    }
+    *cus = c;
+    return HW_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+size_t elem_size(int dtype) { return dtype == HW_F32 ? 4 : 2; }
+
+int validate(const hw_problem* p, int fused) {
+    if (p == nullptr) return HW_ERR_NULL;
+    if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
+    if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
+    if (!(p->scale == p->scale)) return HW_ERR_SHAPE;
+    if (fused) {
+        if (p->RotE < 0 || p->RotE > p->E || (p->RotE & 1)) return HW_ERR_SHAPE;
+    }
+    if (p->out == nullptr || p->q == nullptr || p->locations == nullptr) return HW_ERR_NULL;
+    if (p->k == nullptr || p->v == nullptr || p->len == nullptr) return HW_ERR_NULL;
+    if (fused && p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
+    long long rows = (long long)p->W * p->S * (p->Hq / p->Hkv);
+    if (rows > (1 << 20)) return HW_ERR_SHAPE;
+    for (int f = 0; f < p->F; ++f) {
+        if (p->len[f] < 0) return HW_ERR_SHAPE;
+        if (p->len[f] > 0 && (p->k[f] == nullptr || p->v[f] == nullptr)) return HW_ERR_NULL;
+        if (!aligned16(p->k[f]) || !aligned16(p->v[f])) return HW_ERR_ALIGN;
+        if ((long long)p->len[f] * p->Hkv * p->E * (long long)elem_size(p->dtype) > (1ll << 40)) return HW_ERR_SHAPE;
+    }
+    if (!aligned16(p->out) || !aligned16(p->q)) return HW_ERR_ALIGN;
+    // kernels are instantiated for these head dims (never a silent no-op as in kernel_v21.cuh:992-995)
+    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
+    return HW_OK;
+}
+
+int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
+    if (plan == nullptr) return HW_ERR_NULL;
+    if (num_cus < 1) return HW_ERR_SHAPE;
+    std::memset(plan, 0, sizeof(*plan));
+    const int rows = p->W * p->S * (p->Hq / p->Hkv);
+    plan->rows = rows;
+    plan->row_blocks = rows <= 16 ? 1 : 2;
+    const int rows_per_wg = 16 * plan->row_blocks;
+    plan->row_groups = (rows + rows_per_wg - 1) / rows_per_wg;
+    plan->tile_tokens = hw::TILE;
+    long long tiles = 0;
+    for (int f = 0; f < p->F; ++f) {
+        plan->tile_begin[f] = (int)tiles;
+        tiles += (p->len[f] + hw::TILE - 1) / hw::TILE;
+        if (tiles > (1ll << 30)) return HW_ERR_SHAPE;
+    }
+    for (int f = p->F; f <= HW_MAX_FRAGMENTS; ++f) plan->tile_begin[f] = (int)tiles;
+    plan->tiles_per_head = (int)tiles;
+
+    // Split-K policy: fill every CU with its resident workgroups once, but at least one tile per wave
+    // in every workgroup, and never more workgroups than tiles.
+    int wgs = p->splits;
+    if (wgs <= 0) {
+        // the two-row-block and fp32 kernels are built for one wave per SIMD (one workgroup per CU)
+        const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32) ? 2 : 1;
+        const int target = per_cu * num_cus;
+        wgs = target / (p->Hkv * plan->row_groups);
+        const int by_work = (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
+        if (wgs > by_work) wgs = by_work;
+    }
+    if (wgs > (int)tiles) wgs = (int)tiles;
+    if (wgs < 1) wgs = 1;
+    plan->wgs_per_head = wgs;
+    plan->workgroups = wgs * p->Hkv * plan->row_groups;
+    const size_t parts = (size_t)p->Hkv * wgs;
+    plan->workspace_bytes = parts * rows * ((size_t)p->Ev + 2) * sizeof(float);
+    plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
+    return HW_OK;
+}
+
+int run(const hw_problem* p, void* stream_, int fused) {
+    int st = validate(p, fused);
+    if (st != HW_OK) return st;
+    int cus = 0;
+    st = device_cus(&cus);
+    if (st != HW_OK) return st;
+    hw_plan plan;
+    st = make_plan(p, cus, &plan);
+    if (st != HW_OK) return st;
+    if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
+
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    hw::KernelArgs ka;
+    std::memset(&ka, 0, sizeof(ka));
+    for (int f = 0; f < p->F; ++f) {
+        ka.frag.k[f] = p->k[f];
+        ka.frag.v[f] = p->v[f];
+        ka.frag.len[f] = p->len[f];
+    }
+    for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
+    ka.q = p->q;
+    ka.loc = p->locations;
+    ka.cos = p->cosines;
+    ka.sin = p->sines;
+    ka.rq = fused ? p->rq : nullptr;
+    const size_t parts = (size_t)p->Hkv * plan.wgs_per_head;
+    ka.part_o = reinterpret_cast<float*>(p->workspace);
+    ka.part_ml = ka.part_o + parts * plan.rows * p->Ev;
+    ka.F = p->F; ka.W = p->W; ka.Hq = p->Hq; ka.Hkv = p->Hkv; ka.S = p->S;
+    ka.RotE = fused ? p->RotE : 0;
+    ka.R = plan.rows;
+    ka.nrg = plan.row_groups;
+    ka.wgs_per_head = plan.wgs_per_head;
+    ka.tiles_per_head = plan.tiles_per_head;
+    ka.nwg = plan.workgroups;
+    ka.prerotated = fused ? 0 : 1;
+    ka.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
+    ka.sc = (float)((double)p->scale * 1.4426950408889634074);
+
+    hipError_t e;
+    if (p->ev_start != nullptr) {
+        e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_start), stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, stream);
+    if (e != hipSuccess) return (int)e;
+    if (p->ev_stop != nullptr) {
+        e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_stop), stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    hw::MergeArgs ma;
+    ma.part_o = ka.part_o;
+    ma.part_ml = ka.part_ml;
+    ma.out = p->out;
+    ma.lse = p->lse;
+    ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = plan.rows;
+    ma.wgs_per_head = plan.wgs_per_head;
+    e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
+    return (int)e;
+}
+
+}  // namespace
+
+extern "C" {
+
+int hw_version(void) { return HW_ABI_VERSION; }
+
+const char* hw_status_string(int status) {
+    switch (status) {
+        case HW_OK: return "ok";
+        case HW_ERR_NULL: return "required pointer is NULL";
+        case HW_ERR_DTYPE: return "unknown dtype";
+        case HW_ERR_SHAPE: return "invalid or inconsistent shape";
+        case HW_ERR_UNSUPPORTED: return "no kernel instantiated for this shape (need E == Ev in {64, 128})";
+        case HW_ERR_FRAGMENTS: return "fragment count out of range";
+        case HW_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
+        case HW_ERR_ALIGN: return "device pointer not 16-byte aligned";
+        case HW_ERR_NO_DEVICE: return "no usable HIP device";
+        default: break;
+    }
+    if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
+    return "unknown status";
+}
+
+int hw_validate(const hw_problem* p, int fused) { return validate(p, fused); }
+
+int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan) {
+    // planning needs only the shape and the lengths
+    if (p == nullptr || plan == nullptr || p->len == nullptr) return HW_ERR_NULL;
+    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->Ev < 1 || p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
+    for (int f = 0; f < p->F; ++f)
+        if (p->len[f] < 0) return HW_ERR_SHAPE;
+    return make_plan(p, num_cus, plan);
+}
+
+int hw_workspace_bytes(const hw_problem* p, size_t* bytes) {
+    if (bytes == nullptr) return HW_ERR_NULL;
+    int cus = 0;
+    int st = device_cus(&cus);
+    if (st != HW_OK) return st;
+    hw_plan plan;
+    st = hw_plan_debug(p, cus, &plan);
+    if (st != HW_OK) return st;
+    *bytes = plan.workspace_bytes;
+    return HW_OK;
+}
+
+int hw_fused_attention(const hw_problem* p, void* stream) { return run(p, stream, 1); }
+
+int hw_sdpa(const hw_problem* p, void* stream) { return run(p, stream, 0); }
+
+int hw_rope(void* out, const void* q, const float* cosines, const float* sines, int dtype, int F, int W, int Hq, int S, int E,
+            int RotE, void* stream) {
+    if (out == nullptr || q == nullptr) return HW_ERR_NULL;
+    if (dtype != HW_F32 && dtype != HW_F16 && dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (F < 1 || W < 1 || Hq < 1 || S < 1 || E < 1) return HW_ERR_SHAPE;
+    if (RotE < 0 || RotE > E || (RotE & 1)) return HW_ERR_SHAPE;
+    if (RotE > 0 && (cosines == nullptr || sines == nullptr)) return HW_ERR_NULL;
+    return (int)hw::launch_rope(out, q, cosines, sines, dtype, F, W, Hq, S, E, RotE, reinterpret_cast<hipStream_t>(stream));
+}
+
+int hw_device_cus(void) {
+    int c = 0;
+    return device_cus(&c) == HW_OK ? c : 0;
+}
+
+int hw_event_create(void** ev) {
+    if (ev == nullptr) return HW_ERR_NULL;
+    hipEvent_t e;
+    hipError_t r = hipEventCreate(&e);
+    if (r != hipSuccess) return (int)r;
+    *ev = e;
+    return HW_OK;
+}
+int hw_event_destroy(void* ev) { return ev ? (int)hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)) : HW_ERR_NULL; }
+int hw_event_record(void* ev, void* stream) {
+    return ev ? (int)hipEventRecord(reinterpret_cast<hipEvent_t>(ev), reinterpret_cast<hipStream_t>(stream)) : HW_ERR_NULL;
+}
+int hw_event_synchronize(void* ev) { return ev ? (int)hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)) : HW_ERR_NULL; }
+int hw_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!start || !stop || !ms) return HW_ERR_NULL;
+    return (int)hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop));
+}
+
+int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream) {
+    if (src == nullptr || sink == nullptr) return HW_ERR_NULL;
+    if (bytes % 16 != 0 || !aligned16(src)) return HW_ERR_ALIGN;
+    return (int)hw::launch_stream_read(src, bytes, sink, reinterpret_cast<hipStream_t>(stream));
+}
+
+int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream) {
+    if (src == nullptr || dst == nullptr) return HW_ERR_NULL;
+    if (bytes % 16 != 0 || !aligned16(src) || !aligned16(dst)) return HW_ERR_ALIGN;
+    return (int)hw::launch_stream_copy(dst, src, bytes, reinterpret_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,54 @@
+// Internal interface between the C-ABI host code and the gfx950 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace hw {
+
+constexpr int MAXF = 32;       // fragments per launch (table travels in the kernel arguments)
+constexpr int TILE = 32;       // tokens per wave step
+constexpr int NWAVES = 4;      // waves per workgroup
+constexpr int NTHREADS = NWAVES * 64;
+
+// Fragment table passed by value in the kernel arguments: no per-call host-to-device copy of a pointer
+// table (the reference does one, src/binding.cu:84-103).
+struct FragTable {
+    const void* k[MAXF];
+    const void* v[MAXF];
+    int len[MAXF];
+    int tile_begin[MAXF + 1];   // prefix sum of ceil(len/TILE): position of each fragment in a head's tile sequence
+};
+
+struct KernelArgs {
+    FragTable frag;
+    const void* q;
+    const int* loc;
+    const float* cos;
+    const float* sin;
+    void* rq;
+    float* part_o;      // [Hkv][wgs_per_head][R][Ev]  unnormalised partial outputs
+    float* part_ml;     // [Hkv][wgs_per_head][R][2]   running max (base-2 units) and sum
+    int F, W, Hq, Hkv, S, RotE, R;
+    int nrg, wgs_per_head, tiles_per_head, nwg;
+    int prerotated;
+    int xcd_remap;
+    float sc;           // scale * log2(e)
+};
+
+struct MergeArgs {
+    const float* part_o;
+    const float* part_ml;
+    void* out;
+    float* lse;
+    int W, Hq, Hkv, S, R, wgs_per_head;
+};
+
+hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream);
+hipError_t launch_merge(const MergeArgs& ma, int dtype, int EV, hipStream_t stream);
+hipError_t launch_rope(void* out, const void* q, const float* cosv, const float* sinv, int dtype, int F, int W, int Hq, int S,
+                       int E, int RotE, hipStream_t stream);
+hipError_t launch_stream_read(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
+hipError_t launch_stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
+
+}  // namespace hw
