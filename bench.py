@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Benchmark of the Hogwild! fused decode-attention step on one MI355X.
+
+A "step" is one call of the fused operator (per-fragment q-RoPE + fragmented-KV GQA attention + LSE
+merge) for one decoder layer of the QwQ-32B-shape, 4-worker workload.  Inputs are synthetic, generated
+on the CPU from a fixed seed and resident in HBM before the timed region starts.
+
+Cold-cache protocol: the K/V fragments exist in a ring of distinct copies totalling > 640 MB, and
+consecutive steps walk the ring, so neither the L2 nor the 256 MiB Infinity Cache can serve a repeat.
+
+Prints ONE JSON line.  `value` = algorithmic KV bytes per step / measured time per step, where the K
+steps are replayed from one HIP graph (launch overhead of a Python loop would otherwise dominate a
+~10 us step); the eager-loop figure, the hot-cache figure and a plain streaming-read calibration are
+reported under "extra".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0   # MI355X published HBM3E bandwidth
+METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 workers"
+
+# HBM bytes per launch of the attention kernel on this workload measured with rocprofv3 --pmc
+# (FETCH_SIZE, WRITE_SIZE; scaled by a copy kernel of known size).  None until measured.
+MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--case", type=int, default=3, help="workload configuration 1..5 (3 = headline)")
+    ap.add_argument("--splits", type=int, default=0, help="workgroups per kv head (0 = library default)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
+    ap.add_argument("--ring-mb", type=int, default=640)
+    return ap.parse_args()
+
+
+def make_ring(case, dev, ring_mb):
+    """Distinct device copies of the KV fragments; q / locations / cos / sin are shared (tiny)."""
+    import torch
+    kvb = case.kv_bytes()
+    n = max(2, math.ceil(ring_mb * 1e6 / kvb))
+    ring = []
+    g = torch.Generator().manual_seed(1234)
+    for i in range(n):
+        if i == 0:
+            keys = [k.to(dev) for k in case.keys]
+            vals = [v.to(dev) for v in case.values]
+        else:
+            # same distribution, different bytes: roll along the token axis (cheap, keeps N(0,1) statistics)
+            keys = [torch.roll(k, shifts=i, dims=1).to(dev).contiguous() for k in case.keys]
+            vals = [torch.roll(v, shifts=i, dims=1).to(dev).contiguous() for v in case.values]
+        ring.append((keys, vals))
+    return ring
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the path has no multi-GPU part); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from inference_lib_amd import _lib, cases
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(3)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    case = cases.baseline_case(args.case)
+    kv_bytes = case.kv_bytes()
+    cd = case.to(dev)
+    ring = make_ring(case, dev, args.ring_mb)
+    W, Hq, S, E = cd.q.shape
+    tdt = cd.q.dtype
+
+    out = torch.empty((W, Hq, S, E), dtype=tdt, device=dev)
+    lse = torch.empty((W, Hq, S), dtype=torch.float32, device=dev)
+    rq = None if args.no_rq else torch.empty((case.F, W, Hq, S, E), dtype=tdt, device=dev)
+    problems = []
+    ws = None
+    for keys, vals in ring:
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=out,
+                          cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse, splits=args.splits)
+        if ws is None:
+            ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
+        pr.set_workspace(ws)
+        problems.append(pr)
+    nring = len(problems)
+    plan = _lib.plan(case.lens, W=case.W, S=case.S, Hq=case.Hq, Hkv=case.Hkv, Ev=case.E,
+                     num_cus=_lib.lib.hw_device_cus(), splits=args.splits)
+
+    K, Wm = args.steps, args.warmup
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        # ---------------- eager loop (launch-bound from Python; reported under extra) ----------------
+        for i in range(Wm):
+            problems[i % nring].run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            problems[i % nring].run()
+        torch.cuda.synchronize()
+        eager_us = (time.perf_counter() - t0) / K * 1e6
+
+        # ---------------- HIP graph of exactly K steps walking the ring ----------------
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(K):
+                problems[i % nring].run()
+        for _ in range(max(1, Wm // max(1, K))):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
+        graph_us = (time.perf_counter() - t0) / K * 1e6
+
+        # ---------------- hot cache: the same KV set every step ----------------
+        graph_hot = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph_hot, stream=stream):
+            for i in range(K):
+                problems[0].run()
+        graph_hot.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph_hot.replay()
+        torch.cuda.synchronize()
+        hot_us = (time.perf_counter() - t0) / K * 1e6
+
+        # ---------------- per-launch duration of the attention kernel (HIP events on its stream) ----------------
+        evs = [(_lib.Event(), _lib.Event()) for _ in range(K)]
+        for i in range(min(Wm, 5)):
+            problems[i % nring].run()
+        torch.cuda.synchronize()
+        for i in range(K):
+            pr = problems[i % nring]
+            pr.set_events(evs[i][0].handle, evs[i][1].handle)
+            pr.run()
+            pr.set_events(None, None)
+        torch.cuda.synchronize()
+        durs = sorted(a.elapsed_ms(b) * 1e3 for a, b in evs)
+        kern_us_avg = sum(durs) / len(durs)
+        kern_us_med = durs[len(durs) // 2]
+
+        # ---------------- plain streaming read of the whole ring (achievable HBM rate) ----------------
+        big = torch.empty(int(args.ring_mb * 1e6) // 16 * 16, dtype=torch.uint8, device=dev)
+        big.random_(0, 255)
+        sink = torch.zeros(256, dtype=torch.int32, device=dev)
+        e0, e1 = _lib.Event(), _lib.Event()
+        s_handle = stream.cuda_stream
+        import ctypes as C
+        for _ in range(2):
+            _lib.check(_lib.lib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), C.c_void_p(s_handle)), "hw_stream_read")
+        e0.record(s_handle)
+        for _ in range(5):
+            _lib.check(_lib.lib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), C.c_void_p(s_handle)), "hw_stream_read")
+        e1.record(s_handle)
+        torch.cuda.synchronize()
+        stream_gbs = big.numel() * 5 / (e0.elapsed_ms(e1) * 1e-3) / 1e9
+        del big
+
+    value = kv_bytes / (graph_us * 1e-6) / 1e9
+    achieved = kv_bytes / (kern_us_avg * 1e-6) / 1e9
+    result = {
+        "metric": METRIC,
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": Wm,
+        "ms_per_step": round(graph_us * 1e-3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": case.dtype,
+        "data": "synthetic",
+        "config": {
+            "workload": f"config {args.case} ({case.name}): W={case.W} S={case.S} Hq={case.Hq} Hkv={case.Hkv} D={case.E} "
+                        f"{case.dtype}, fragments={case.lens}",
+            "kv_bytes_per_step": kv_bytes,
+            "visible_tokens": case.visible_tokens(),
+            "cold_cache_ring_sets": nring,
+            "workgroups": plan.workgroups,
+            "wgs_per_head": plan.wgs_per_head,
+            "writes_rotated_q": rq is not None,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(case.name),
+            "kernel": "hw::attention_kernel",
+            "kernel_us_avg": round(kern_us_avg, 3),
+            "kernel_us_median": round(kern_us_med, 3),
+        },
+        "extra": {
+            "us_per_step": round(graph_us, 3),
+            "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2),
+            "eager_loop_us_per_step": round(eager_us, 3),
+            "hot_cache_us_per_step": round(hot_us, 3),
+            "hot_cache_GBps": round(kv_bytes / (hot_us * 1e-6) / 1e9, 1),
+            "stream_read_GBps": round(stream_gbs, 1),
+            "timing": "K steps replayed as one HIP graph, wall clock between device synchronisations",
+        },
+    }
+
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(case, kv_bytes)
+    print(json.dumps(result, ensure_ascii=False))
+
+
+def cpu_baseline(case, kv_bytes):
+    """The reference's eager PyTorch path (python/hogwild/attention.py:38-67 + :84-90) restated in
+    oracle/, timed on the host cores of this box.  Baseline only."""
+    import torch
+    from oracle import hogwild_oracle as O
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    args = (case.q, case.locations, case.keys, case.values, case.scale, case.cos, case.sin)
+    for _ in range(2):
+        O.torch_reference_step(*args)
+    ts = []
+    t_all = time.perf_counter()
+    while len(ts) < 10 and (time.perf_counter() - t_all) < 30.0:
+        t0 = time.perf_counter()
+        O.torch_reference_step(*args)
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    med = ts[len(ts) // 2]
+    return {
+        "value": round(kv_bytes / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "us_per_step": round(med * 1e6, 1),
+        "sample": f"{len(ts)} full steps of the same workload (median), torch fp32 eager restatement of the reference path",
+    }
+
+
+if __name__ == "__main__":
+    main()

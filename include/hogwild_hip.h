@@ -28,6 +28,7 @@ extern "C" {
 
 #define HW_ABI_VERSION 1
 #define HW_MAX_FRAGMENTS 32
+#define HW_MAX_SPLITS 256      /* workgroups per kv head */
 
 typedef enum hw_status {
     HW_OK = 0,
@@ -92,7 +93,9 @@ typedef struct hw_plan {
     int32_t tiles_per_head;   /* sum_f ceil(len[f] / tile_tokens) */
     int32_t wgs_per_head;     /* split-K factor */
     int32_t workgroups;       /* grid size of the attention kernel */
-    int32_t tile_begin[HW_MAX_FRAGMENTS + 1];
+    int32_t tile_begin[HW_MAX_FRAGMENTS + 1];   /* first tile of each fragment in a head's tile sequence */
+    int32_t wg_tile_begin[HW_MAX_SPLITS + 1];   /* first tile of each workgroup; balanced by tiles + a fixed
+                                                    cost for every fragment a workgroup has to open */
     size_t workspace_bytes;
 } hw_plan;
 

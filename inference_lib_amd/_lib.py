@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
 
 HW_MAX_FRAGMENTS = 32
+HW_MAX_SPLITS = 256
 HW_F32, HW_F16, HW_BF16 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_BF16}
 
@@ -47,6 +48,7 @@ class HwPlan(C.Structure):
         ("rows", C.c_int32), ("row_blocks", C.c_int32), ("row_groups", C.c_int32), ("tile_tokens", C.c_int32),
         ("tiles_per_head", C.c_int32), ("wgs_per_head", C.c_int32), ("workgroups", C.c_int32),
         ("tile_begin", C.c_int32 * (HW_MAX_FRAGMENTS + 1)),
+        ("wg_tile_begin", C.c_int32 * (HW_MAX_SPLITS + 1)),
         ("workspace_bytes", C.c_size_t),
     ]
 

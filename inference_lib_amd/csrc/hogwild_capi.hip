@@ -58,6 +58,7 @@ int validate(const hw_problem* p, int fused) {
         if ((long long)p->len[f] * p->Hkv * p->E * (long long)elem_size(p->dtype) > (1ll << 40)) return HW_ERR_SHAPE;
     }
     if (!aligned16(p->out) || !aligned16(p->q)) return HW_ERR_ALIGN;
+    if (fused && (!aligned16(p->cosines) || !aligned16(p->sines) || !aligned16(p->rq))) return HW_ERR_ALIGN;
     // kernels are instantiated for these head dims (never a silent no-op as in kernel_v21.cuh:992-995)
     if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
     return HW_OK;
@@ -94,7 +95,52 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
         if (wgs > by_work) wgs = by_work;
     }
     if (wgs > (int)tiles) wgs = (int)tiles;
+    if (wgs > hw::MAX_SPLITS) wgs = hw::MAX_SPLITS;
     if (wgs < 1) wgs = 1;
+
+    // Workgroup boundaries.  Opening a fragment costs a workgroup a fixed prologue (query rotation, a
+    // barrier, a pipeline refill) worth about kOpenCost tiles, so boundaries balance tiles + openings
+    // rather than tiles alone: a run of tiny fragments is spread over several workgroups instead of
+    // serialising their prologues in one straggler.
+    {
+        const double kOpenCost = 6.0;
+        int nfrag_left = 0;
+        for (int f = 0; f < p->F; ++f) nfrag_left += p->len[f] > 0 ? 1 : 0;
+        long long tiles_left = tiles;
+        int wg = 0;
+        double used = 0.0;
+        plan->wg_tile_begin[0] = 0;
+        for (int f = 0; f < p->F; ++f) {
+            const int ft = (p->len[f] + hw::TILE - 1) / hw::TILE;
+            if (ft == 0) continue;
+            int t = 0;
+            while (t < ft) {
+                const int wgs_left = wgs - wg;   // including the current one
+                // fair share of what remains, counting one opening per remaining fragment and workgroup
+                const double remaining = (double)tiles_left + kOpenCost * (nfrag_left + wgs_left - 1) + used;
+                const double target = remaining / wgs_left;
+                const double room = target - used - kOpenCost;
+                if (room < 1.0 && used > 0.0 && wgs_left > 1) {   // not worth opening this fragment here
+                    plan->wg_tile_begin[++wg] = plan->tile_begin[f] + t;
+                    used = 0.0;
+                    continue;
+                }
+                int take = (int)(room + 0.5);
+                if (take < 1) take = 1;
+                if (take > ft - t || wgs_left == 1) take = ft - t;
+                used += kOpenCost + take;
+                t += take;
+                tiles_left -= take;
+                if (t < ft) {   // the fragment continues in the next workgroup
+                    plan->wg_tile_begin[++wg] = plan->tile_begin[f] + t;
+                    used = 0.0;
+                }
+            }
+            --nfrag_left;
+        }
+        wgs = tiles > 0 ? wg + 1 : 1;
+        for (int i = wgs; i <= HW_MAX_SPLITS; ++i) plan->wg_tile_begin[i] = (int)tiles;
+    }
     plan->wgs_per_head = wgs;
     plan->workgroups = wgs * p->Hkv * plan->row_groups;
     const size_t parts = (size_t)p->Hkv * wgs;
@@ -123,24 +169,25 @@ int run(const hw_problem* p, void* stream_, int fused) {
         ka.frag.len[f] = p->len[f];
     }
     for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
-    ka.q = p->q;
-    ka.loc = p->locations;
-    ka.cos = p->cosines;
-    ka.sin = p->sines;
-    ka.rq = fused ? p->rq : nullptr;
+    for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];
+    ka.h.q = p->q;
+    ka.h.loc = p->locations;
+    ka.h.cos = p->cosines;
+    ka.h.sin = p->sines;
+    ka.h.rq = fused ? p->rq : nullptr;
     const size_t parts = (size_t)p->Hkv * plan.wgs_per_head;
-    ka.part_o = reinterpret_cast<float*>(p->workspace);
-    ka.part_ml = ka.part_o + parts * plan.rows * p->Ev;
-    ka.F = p->F; ka.W = p->W; ka.Hq = p->Hq; ka.Hkv = p->Hkv; ka.S = p->S;
-    ka.RotE = fused ? p->RotE : 0;
-    ka.R = plan.rows;
-    ka.nrg = plan.row_groups;
-    ka.wgs_per_head = plan.wgs_per_head;
-    ka.tiles_per_head = plan.tiles_per_head;
-    ka.nwg = plan.workgroups;
-    ka.prerotated = fused ? 0 : 1;
-    ka.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
-    ka.sc = (float)((double)p->scale * 1.4426950408889634074);
+    ka.h.part_o = reinterpret_cast<float*>(p->workspace);
+    ka.h.part_ml = ka.h.part_o + parts * plan.rows * p->Ev;
+    ka.h.F = p->F; ka.h.W = p->W; ka.h.Hq = p->Hq; ka.h.Hkv = p->Hkv; ka.h.S = p->S;
+    ka.h.RotE = fused ? p->RotE : 0;
+    ka.h.R = plan.rows;
+    ka.h.nrg = plan.row_groups;
+    ka.h.wgs_per_head = plan.wgs_per_head;
+    ka.h.tiles_per_head = plan.tiles_per_head;
+    ka.h.nwg = plan.workgroups;
+    ka.h.prerotated = fused ? 0 : 1;
+    ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
+    ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
 
     hipError_t e;
     if (p->ev_start != nullptr) {
@@ -154,8 +201,8 @@ int run(const hw_problem* p, void* stream_, int fused) {
         if (e != hipSuccess) return (int)e;
     }
     hw::MergeArgs ma;
-    ma.part_o = ka.part_o;
-    ma.part_ml = ka.part_ml;
+    ma.part_o = ka.h.part_o;
+    ma.part_ml = ka.h.part_ml;
     ma.out = p->out;
     ma.lse = p->lse;
     ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = plan.rows;

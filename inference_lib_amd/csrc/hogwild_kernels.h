@@ -10,6 +10,7 @@ constexpr int MAXF = 32;       // fragments per launch (table travels in the ker
 constexpr int TILE = 32;       // tokens per wave step
 constexpr int NWAVES = 4;      // waves per workgroup
 constexpr int NTHREADS = NWAVES * 64;
+constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary table below)
 
 // Fragment table passed by value in the kernel arguments: no per-call host-to-device copy of a pointer
 // table (the reference does one, src/binding.cu:84-103).
@@ -20,8 +21,9 @@ struct FragTable {
     int tile_begin[MAXF + 1];   // prefix sum of ceil(len/TILE): position of each fragment in a head's tile sequence
 };
 
-struct KernelArgs {
-    FragTable frag;
+// Scalar arguments of the attention kernel: exactly 32 dwords at the start of the kernel-argument segment
+// so that the kernel can fetch all of them with two back-to-back 64-byte scalar loads.
+struct alignas(64) KernelHeader {
     const void* q;
     const int* loc;
     const float* cos;
@@ -34,6 +36,14 @@ struct KernelArgs {
     int prerotated;
     int xcd_remap;
     float sc;           // scale * log2(e)
+    int pad[4];
+};
+static_assert(sizeof(KernelHeader) == 128, "KernelHeader must be 32 dwords");
+
+struct KernelArgs {
+    KernelHeader h;
+    FragTable frag;
+    int wg_tile[MAX_SPLITS + 1];   // first tile of each workgroup of a head (same for all heads)
 };
 
 struct MergeArgs {

@@ -26,6 +26,18 @@
 
 namespace hw {
 
+// Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
+#ifdef HW_CLOCKS
+__device__ unsigned long long hw_clock_buf[4096 * 8];
+#define HW_MARK(i)                                                                                  \
+    do {                                                                                            \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
+            hw_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();         \
+    } while (0)
+#else
+#define HW_MARK(i) do { } while (0)
+#endif
+
 typedef unsigned int u32;
 typedef u32 u32x2 __attribute__((ext_vector_type(2)));
 typedef u32 u32x4 __attribute__((ext_vector_type(4)));
@@ -103,7 +115,11 @@ __device__ __forceinline__ int slot_token(int q, int idx) { return ((idx >> 2) <
 template <class DT, int E, int EV>
 struct Geo {
     static constexpr int SZ = Elem<DT>::size;
-    static constexpr int KJ = E * SZ / 64;               // 16-byte K loads per lane per 16-token block
+    static constexpr int KJ = E * SZ / 64;               // 16-byte K operand chunks per lane per 16-token block
+    static constexpr int KROW = E * SZ;                  // bytes of one K row
+    static constexpr int CPR = KROW / 16;                // 16-byte chunks per K row
+    static constexpr int KL = TILE * KROW / 1024;        // 1 KB wave-wide K loads per tile
+    static constexpr int KSTAGE = TILE * KROW;           // bytes of the per-wave K staging area in LDS
     static constexpr int VW = EV * SZ / 64;              // dwords of one V row held by one lane
     static constexpr int VLD = VW < 4 ? VW : 4;          // dwords per V load
     static constexpr int NVL = VW / VLD;                 // V loads per row per lane
@@ -115,42 +131,60 @@ struct Geo {
 template <class DT, int E, int EV>
 struct TileRegs {
     typedef Geo<DT, E, EV> G;
-    u32x4 k[2][G::KJ];
+    u32x4 k[G::KL];      // the tile's K rows as one contiguous stream: load i, lane l holds chunk i*64 + l
     u32 v[8][G::VW];
 };
 
+// K/V fragment pointers arrive as integers out of the fragment table; they are given the global address
+// space explicitly so that the tile loads are global_load (vmcnt only), not flat_load.
+typedef const __attribute__((address_space(1))) char* gptr_t;
+
 template <class DT, int E, int EV>
-__device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const char* kbase, const char* vbase, int t0, int L,
-                                          int n, int q) {
+__device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, gptr_t kbase, gptr_t vbase, int t0, int L, int n, int q,
+                                          bool real) {
     typedef Geo<DT, E, EV> G;
-    const int last = L - 1;
+    // A tile past the end of the segment is still "loaded" so that the number of loads in flight is the same
+    // on every path (the wait counts then stay exact instead of draining everything); all its lanes read the
+    // first 16 bytes of the fragment, which costs one cache line.
+    const int last = real ? L - 1 : 0;
+    if (!real) t0 = 0, n = 0, q = 0;
+    const int lane = q * 16 + n;
+    // K: consecutive lanes read consecutive 16-byte chunks, so each load covers 1 KB of contiguous rows
 #pragma unroll
-    for (int tb = 0; tb < 2; ++tb) {
-        int tok = min(t0 + tb * 16 + n, last);
-        const char* row = kbase + (size_t)tok * (E * G::SZ);
-#pragma unroll
-        for (int j = 0; j < G::KJ; ++j) t.k[tb][j] = *reinterpret_cast<const u32x4*>(row + (4 * j + q) * 16);
+    for (int i = 0; i < G::KL; ++i) {
+        const int g = real ? i * 64 + lane : 0;
+        const int tok = min(t0 + g / G::CPR, last);
+        t.k[i] = *reinterpret_cast<const __attribute__((address_space(1))) u32x4*>(kbase + (size_t)tok * G::KROW + (g % G::CPR) * 16);
     }
 #pragma unroll
     for (int idx = 0; idx < 8; ++idx) {
         int tok = min(t0 + slot_token(q, idx), last);
-        const char* row = vbase + (size_t)tok * (EV * G::SZ);
+        gptr_t row = vbase + (size_t)tok * (EV * G::SZ);
 #pragma unroll
         for (int hh = 0; hh < G::NVL; ++hh) {
-            const char* p = row + hh * 256 + n * (G::VLD * 4);
+            gptr_t p = row + hh * 256 + n * (G::VLD * 4);
             if constexpr (G::VLD == 4) {
-                u32x4 x = *reinterpret_cast<const u32x4*>(p);
+                u32x4 x = *reinterpret_cast<const __attribute__((address_space(1))) u32x4*>(p);
                 t.v[idx][hh * 4 + 0] = x.x;
                 t.v[idx][hh * 4 + 1] = x.y;
                 t.v[idx][hh * 4 + 2] = x.z;
                 t.v[idx][hh * 4 + 3] = x.w;
             } else {
-                u32x2 x = *reinterpret_cast<const u32x2*>(p);
+                u32x2 x = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(p);
                 t.v[idx][0] = x.x;
                 t.v[idx][1] = x.y;
             }
         }
     }
+}
+
+// LDS position of 16-byte chunk c of tile row `row` in the per-wave K staging area.  The xor key makes both
+// the coalesced write (16 consecutive lanes = consecutive chunks) and the operand read (16 lanes = 16
+// different rows, same chunk) touch 16 different 16-byte bank groups.
+template <class G>
+__device__ __forceinline__ int kstage_offset(int row, int c) {
+    const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+    return row * G::KROW + ((c ^ key) << 4);
 }
 
 // Running state of one wave: RB row blocks of 16 rows each.
@@ -163,9 +197,28 @@ struct WaveState {
 
 template <class DT, int E, int EV, int RB>
 __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const u32x4 (&qreg)[RB][Geo<DT, E, EV>::KJ],
-                                             const int (&lim)[RB], WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int q,
-                                             float sc) {
+                                             const int (&lim)[RB], WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q,
+                                             float sc, char* kstage) {
     typedef Geo<DT, E, EV> G;
+    // K: registers (stream order) -> LDS -> registers in MFMA A-operand order (lane = token, 16 B of head dim).
+    // The staging area is private to the wave and LDS executes a wave's instructions in order.
+    {
+        const int lane = q * 16 + n;
+#pragma unroll
+        for (int i = 0; i < G::KL; ++i) {
+            const int g = i * 64 + lane;
+            *reinterpret_cast<u32x4*>(kstage + kstage_offset<G>(g / G::CPR, g % G::CPR)) = t.k[i];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    u32x4 kop[2][G::KJ];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+#pragma unroll
+        for (int j = 0; j < G::KJ; ++j)
+            kop[tb][j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
+    }
+    __builtin_amdgcn_wave_barrier();
     float p[RB][8];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -175,13 +228,13 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
             if constexpr (G::SZ == 2) {
 #pragma unroll
-                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(t.k[tb][j], qreg[rb][j], acc);
+                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[tb][j], qreg[rb][j], acc);
             } else {
 #pragma unroll
                 for (int j = 0; j < G::KJ; ++j) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c)
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(t.k[tb][j][c]), __uint_as_float(qreg[rb][j][c]),
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(kop[tb][j][c]), __uint_as_float(qreg[rb][j][c]),
                                                                    acc, 0, 0, 0);
                 }
             }
@@ -262,10 +315,200 @@ __device__ __forceinline__ int out_ev(int c, int i) {
     }
 }
 
+// 16-byte chunk of CH elements <-> CH floats
+template <class DT> struct Chunk;
+template <> struct Chunk<F32> {
+    static constexpr int CH = 4;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(x[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[4]) {
+        return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    }
+};
+template <> struct Chunk<BF16> {
+    static constexpr int CH = 8;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(x[i] << 16);
+            f[2 * i + 1] = __uint_as_float(x[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        return u32x4{Elem<BF16>::pack2(f[0], f[1]), Elem<BF16>::pack2(f[2], f[3]), Elem<BF16>::pack2(f[4], f[5]),
+                     Elem<BF16>::pack2(f[6], f[7])};
+    }
+};
+template <> struct Chunk<F16> {
+    static constexpr int CH = 8;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[8]) {
+        f16x8 h = __builtin_bit_cast(f16x8, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        return u32x4{Elem<F16>::pack2(f[0], f[1]), Elem<F16>::pack2(f[2], f[3]), Elem<F16>::pack2(f[4], f[5]),
+                     Elem<F16>::pack2(f[6], f[7])};
+    }
+};
+
+#define HW_GLOBAL __attribute__((address_space(1)))
+
+// KernelHeader as the kernel sees it after fetching it by hand: same layout, pointers typed as global memory
+// (a pointer rebuilt from raw bits would otherwise be a flat pointer, and flat loads tie up both wait counters).
+struct DevHeader {
+    const HW_GLOBAL char* q;
+    const HW_GLOBAL int* loc;
+    const HW_GLOBAL float* cos;
+    const HW_GLOBAL float* sin;
+    HW_GLOBAL char* rq;
+    HW_GLOBAL float* part_o;
+    HW_GLOBAL float* part_ml;
+    int F, W, Hq, Hkv, S, RotE, R;
+    int nrg, wgs_per_head, tiles_per_head, nwg;
+    int prerotated;
+    int xcd_remap;
+    float sc;
+    int pad[4];
+};
+static_assert(sizeof(DevHeader) == sizeof(KernelHeader), "DevHeader mirrors KernelHeader");
+
+// row r (0..R) of a kv head -> (worker*S + token, q head, flat q row index)
+struct RowMap {
+    int ws;
+    size_t qrow;
+};
+__device__ __forceinline__ RowMap map_row(const DevHeader& a, int r, int hkv, int GQ) {
+    RowMap m;
+    m.ws = r / GQ;
+    const int gq = r - m.ws * GQ;
+    const int w = m.ws / a.S, s = m.ws - w * a.S;
+    m.qrow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
+    return m;
+}
+
+// Query rotation of one fragment, split in two phases so that its few global loads can be issued BEFORE the
+// K/V tile loads (loads return in issue order, so a dependent wait would otherwise drain the whole KV
+// prefetch first) and consumed after them.  One work item = one 16-byte chunk pair (e, e + RotE/2) of one
+// row, or one pass-through chunk.  Index convention of src/rope.cuh:18-51: both halves read cos/sin at the
+// first-half index.  Rotary widths that are not a multiple of two chunks take the scalar path in phase two.
+template <class DT, int E, int ROWS, int QSTR>
+struct QueryRotation {
+    typedef typename Elem<DT>::store_t store_t;
+    static constexpr int SZ = Elem<DT>::size;
+    static constexpr int CH = Chunk<DT>::CH;
+    static constexpr int NIT = (ROWS * (E / CH) + NTHREADS - 1) / NTHREADS;   // items per thread, worst case (no rotation)
+
+    u32x4 xa[NIT], xb[NIT];
+    f32x4 cs[NIT][CH / 4], sn[NIT][CH / 4];
+
+    static __device__ __forceinline__ bool vec_ok(int rot) { return (rot % (2 * CH)) == 0; }
+
+    __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid) {
+        const int rot = a.prerotated ? 0 : a.RotE;
+        if (!vec_ok(rot)) return;
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+        const int npair = (rot / 2) / CH;
+        const int ipr = npair + (E - rot) / CH;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / ipr, slot = item - rr * ipr;
+            const int r = r0 + rr;
+            if (item >= ROWS * ipr || r >= a.R) continue;
+            const RowMap rm = map_row(a, r, hkv, GQ);
+            const HW_GLOBAL char* qp = a.q + (rm.qrow * E + (a.prerotated ? f * fstride : 0)) * SZ;
+            if (slot < npair) {
+                xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
+                xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + npair) * 16);
+                const size_t co = ((size_t)f * a.W * a.S + rm.ws) * a.RotE + slot * CH;
+#pragma unroll
+                for (int i = 0; i < CH / 4; ++i) {
+                    cs[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.cos + co + 4 * i);
+                    sn[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.sin + co + 4 * i);
+                }
+            } else {
+                xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + npair) * 16);
+            }
+        }
+    }
+
+    __device__ __forceinline__ void finish(const DevHeader& a, char* q_lds, int f, int hkv, int r0, int GQ, bool write_rq,
+                                           int tid) const {
+        const int rot = a.prerotated ? 0 : a.RotE;
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+        if (vec_ok(rot)) {
+            const int npair = (rot / 2) / CH;
+            const int ipr = npair + (E - rot) / CH;
+#pragma unroll
+            for (int it = 0; it < NIT; ++it) {
+                const int item = tid + it * NTHREADS;
+                const int rr = item / ipr, slot = item - rr * ipr;
+                const int r = r0 + rr;
+                if (item >= ROWS * ipr) continue;
+                char* lrow = q_lds + rr * QSTR;
+                if (r >= a.R) {   // padding rows of the 16-row MFMA block
+                    const u32x4 z = {0, 0, 0, 0};
+                    if (slot < npair) *reinterpret_cast<u32x4*>(lrow + slot * 16) = z;
+                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = z;
+                    continue;
+                }
+                const RowMap rm = map_row(a, r, hkv, GQ);
+                HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
+                if (slot < npair) {
+                    float x1[CH], x2[CH], y1[CH], y2[CH];
+                    Chunk<DT>::unpack(xa[it], x1);
+                    Chunk<DT>::unpack(xb[it], x2);
+#pragma unroll
+                    for (int i = 0; i < CH; ++i) {
+                        const float c = cs[it][i >> 2][i & 3], sv = sn[it][i >> 2][i & 3];
+                        y1[i] = x1[i] * c - x2[i] * sv;
+                        y2[i] = x2[i] * c + x1[i] * sv;
+                    }
+                    const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
+                    *reinterpret_cast<u32x4*>(lrow + slot * 16) = ya;
+                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = yb;
+                    if (write_rq) {
+                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
+                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + npair) * 16) = yb;
+                    }
+                } else {
+                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = xa[it];
+                    if (write_rq) *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + npair) * 16) = xa[it];
+                }
+            }
+        } else {
+            const int h = rot >> 1;
+            for (int idx = tid; idx < ROWS * E; idx += NTHREADS) {
+                const int rr = idx / E, e = idx - rr * E;
+                const int r = r0 + rr;
+                store_t sv = Elem<DT>::from_float(0.f);
+                if (r < a.R) {
+                    const RowMap rm = map_row(a, r, hkv, GQ);
+                    const HW_GLOBAL store_t* qp = reinterpret_cast<const HW_GLOBAL store_t*>(a.q) + rm.qrow * E;
+                    const float x = Elem<DT>::to_float(qp[e]);
+                    float val = x;
+                    if (e < rot) {
+                        const size_t co = ((size_t)f * a.W * a.S + rm.ws) * a.RotE;
+                        if (e < h) val = x * a.cos[co + e] - Elem<DT>::to_float(qp[e + h]) * a.sin[co + e];
+                        else val = x * a.cos[co + e - h] + Elem<DT>::to_float(qp[e - h]) * a.sin[co + e - h];
+                    }
+                    sv = Elem<DT>::from_float(val);
+                    if (write_rq) reinterpret_cast<HW_GLOBAL store_t*>(a.rq)[(f * fstride + rm.qrow * E) + e] = sv;
+                }
+                *reinterpret_cast<store_t*>(q_lds + rr * QSTR + e * SZ) = sv;
+            }
+        }
+    }
+};
+
 // MINW = waves per SIMD the register budget is sized for: 2 (<= 256 VGPRs) when one 16-row block is live,
-// 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the double-buffered tile registers too large.
-template <class DT, int E, int EV, int RB, int MINW>
-__global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelArgs a) {
+// 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the tile registers too large.
+// PF = tiles a wave keeps in flight.
+template <class DT, int E, int EV, int RB, int MINW, int PF>
+__global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     typedef typename Elem<DT>::store_t store_t;
     constexpr int ROWS = RB * 16;
@@ -274,13 +517,46 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     __shared__ __attribute__((aligned(16))) char q_lds[ROWS * G::QSTR];
     __shared__ int lim_lds[ROWS];
     __shared__ float m_lds[NWAVES][ROWS];
-    __shared__ __attribute__((aligned(16))) float x_lds[2][NREG][64];
+    // wave-exchange buffers of the epilogue, aliased with the per-wave K staging areas of the main loop
+    constexpr int XBYTES = 2 * NREG * 64 * 4;
+    constexpr int SBYTES = NWAVES * G::KSTAGE;
+    __shared__ __attribute__((aligned(16))) char xs_lds[XBYTES > SBYTES ? XBYTES : SBYTES];
+    float (*x_lds)[NREG][64] = reinterpret_cast<float (*)[NREG][64]>(xs_lds);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int q = lane >> 4;
+    char* kstage = xs_lds + wv * G::KSTAGE;
+
+    // Everything the kernel needs from its arguments is requested here in one burst, before anything waits:
+    // the 32 scalar dwords with two 64-byte scalar loads, the fragment table and the workgroup boundary table
+    // with one vector load per lane and array.  The argument segment is slow to reach and the compiler would
+    // otherwise fetch it lazily, one dependent round trip after another.
+    const int fl = lane & (MAXF - 1);
+    const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
+    const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
+    const int my_len = args.frag.len[fl];
+    const int my_tb = args.frag.tile_begin[fl];
+    const int my_te = args.frag.tile_begin[fl + 1];
+    int my_wt[MAX_SPLITS / 64], my_wt1[MAX_SPLITS / 64];
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        my_wt[i] = args.wg_tile[lane + 64 * i];
+        my_wt1[i] = args.wg_tile[lane + 64 * i + 1];
+    }
+    typedef int i32x16 __attribute__((ext_vector_type(16)));
+    struct HeaderBits { i32x16 lo, hi; };
+    HeaderBits hb;
+    {
+        const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
+                     : "=&s"(hb.lo), "=&s"(hb.hi)
+                     : "s"(argp)
+                     : "memory");
+    }
+    const DevHeader a = __builtin_bit_cast(DevHeader, hb);
 
     // consecutive logical ids stay on one XCD (hardware deals workgroups round-robin over the 8 XCDs)
     int bid = blockIdx.x;
@@ -289,11 +565,18 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     const int g = (bid / a.nrg) % a.wgs_per_head;
     const int hkv = bid / (a.nrg * a.wgs_per_head);
 
-    const int T0 = (int)(((long long)g * a.tiles_per_head) / a.wgs_per_head);
-    const int T1 = (int)(((long long)(g + 1) * a.tiles_per_head) / a.wgs_per_head);
+    int T0 = 0, T1 = 0;
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        if ((g >> 6) == i) {   // uniform
+            T0 = __builtin_amdgcn_readlane(my_wt[i], g & 63);
+            T1 = __builtin_amdgcn_readlane(my_wt1[i], g & 63);
+        }
+    }
     const int r0 = rg * ROWS;
     const int GQ = a.Hq / a.Hkv;
 
+    HW_MARK(0);
     WaveState<RB, G::NOC> st;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -303,68 +586,40 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-    for (int f = 0; f < a.F; ++f) {
-        const int fb = a.frag.tile_begin[f];
-        const int fe = a.frag.tile_begin[f + 1];
+    unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
+
+    while (todo != 0) {
+        const int f = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int fb = __builtin_amdgcn_readlane(my_tb, f);
+        const int fe = __builtin_amdgcn_readlane(my_te, f);
         const int s0 = max(T0, fb), s1 = min(T1, fe);
-        if (s0 >= s1) continue;   // uniform over the workgroup
-        const int L = a.frag.len[f];
-        const char* kbase = reinterpret_cast<const char*>(a.frag.k[f]) + (size_t)hkv * L * (E * G::SZ);
-        const char* vbase = reinterpret_cast<const char*>(a.frag.v[f]) + (size_t)hkv * L * (EV * G::SZ);
+        const int L = __builtin_amdgcn_readlane(my_len, f);
+        const unsigned long long kp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_k >> 32), f) << 32) |
+                                      (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
+        const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
+                                      (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
+        gptr_t kbase = (gptr_t)(kp + (unsigned long long)hkv * L * (E * G::SZ));
+        gptr_t vbase = (gptr_t)(vp + (unsigned long long)hkv * L * (EV * G::SZ));
         const int lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
         const int lt1 = s1 - fb;
 
-        TileRegs<DT, E, EV> ta, tb;
-        if (lt0 < lt1) load_tile<DT, E, EV>(ta, kbase, vbase, lt0 * TILE, L, n, q);
-        if (lt0 + NWAVES < lt1) load_tile<DT, E, EV>(tb, kbase, vbase, (lt0 + NWAVES) * TILE, L, n, q);
+        // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first PF
+        // K/V tiles; the rotation then waits only for the former while the tiles stay in flight
+        QueryRotation<DT, E, ROWS, G::QSTR> qrot;
+        qrot.load(a, f, hkv, r0, GQ, tid);
+        // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
+        const int lm = a.loc[(size_t)f * a.W * a.S + min(r0 + (tid & (ROWS - 1)), a.R - 1) / GQ];
+        TileRegs<DT, E, EV> tr[PF];
+#pragma unroll
+        for (int i = 0; i < PF; ++i)
+            load_tile<DT, E, EV>(tr[i], kbase, vbase, (lt0 + i * NWAVES) * TILE, L, n, q, lt0 + i * NWAVES < lt1);
 
+        HW_MARK(1);
         // ---- prologue: rotate the queries of this fragment into LDS ----
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
-        const bool write_rq = a.rq != nullptr && s0 == fb;
-        for (int idx = tid; idx < ROWS * E; idx += NTHREADS) {
-            const int rr = idx / E, e = idx - rr * E;
-            const int r = r0 + rr;
-            float val = 0.f;
-            if (r < a.R) {
-                const int ws = r / GQ, gq = r - ws * GQ;      // ws = w*S + s
-                const int w = ws / a.S, s = ws - w * a.S;
-                const size_t qrow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
-                const store_t* qp = reinterpret_cast<const store_t*>(a.q) + qrow * E;
-                if (a.prerotated) {
-                    val = Elem<DT>::to_float(qp[(size_t)f * a.W * a.Hq * a.S * E + e]);
-                } else {
-                    const float x = Elem<DT>::to_float(qp[e]);
-                    const int h = a.RotE >> 1;
-                    if (e < a.RotE) {
-                        const size_t cs = ((size_t)(f * a.W + w) * a.S + s) * a.RotE;
-                        if (e < h) {
-                            const float x2 = Elem<DT>::to_float(qp[e + h]);
-                            val = x * a.cos[cs + e] - x2 * a.sin[cs + e];
-                        } else {
-                            const float x1 = Elem<DT>::to_float(qp[e - h]);
-                            val = x * a.cos[cs + e - h] + x1 * a.sin[cs + e - h];
-                        }
-                    } else {
-                        val = x;
-                    }
-                }
-                const store_t sv = Elem<DT>::from_float(val);
-                *reinterpret_cast<store_t*>(q_lds + rr * G::QSTR + e * G::SZ) = sv;
-                if (write_rq)
-                    reinterpret_cast<store_t*>(a.rq)[((size_t)f * a.W * a.Hq * a.S + qrow) * E + e] = sv;
-            } else {
-                *reinterpret_cast<store_t*>(q_lds + rr * G::QSTR + e * G::SZ) = Elem<DT>::from_float(0.f);
-            }
-        }
-        if (tid < ROWS) {
-            const int r = r0 + tid;
-            int lm = 0;
-            if (r < a.R) {
-                const int ws = r / GQ;
-                lm = min(L, max(0, a.loc[(size_t)f * a.W * a.S + ws] + 1));
-            }
-            lim_lds[tid] = lm;
-        }
+        qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && s0 == fb, tid);
+        if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0;
         __syncthreads();
 
         u32x4 qreg[RB][G::KJ];
@@ -381,18 +636,20 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 #pragma unroll
         for (int off = 1; off < 16; off <<= 1) maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
         maxlim = __builtin_amdgcn_readfirstlane(maxlim);
+        HW_MARK(2);
 
-        // ---- stream this wave's tiles, two in flight ----
-        for (int lt = lt0; lt < lt1; lt += 2 * NWAVES) {
-            if (lt * TILE < maxlim) compute_tile<DT, E, EV, RB>(ta, qreg, lim, st, lt * TILE, q, a.sc);
-            if (lt + 2 * NWAVES < lt1) load_tile<DT, E, EV>(ta, kbase, vbase, (lt + 2 * NWAVES) * TILE, L, n, q);
-            if (lt + NWAVES < lt1) {
-                if ((lt + NWAVES) * TILE < maxlim) compute_tile<DT, E, EV, RB>(tb, qreg, lim, st, (lt + NWAVES) * TILE, q, a.sc);
-                if (lt + 3 * NWAVES < lt1) load_tile<DT, E, EV>(tb, kbase, vbase, (lt + 3 * NWAVES) * TILE, L, n, q);
+        // ---- stream this wave's tiles, PF in flight ----
+        for (int lt = lt0; lt < lt1; lt += PF * NWAVES) {
+#pragma unroll
+            for (int i = 0; i < PF; ++i) {
+                const int l = lt + i * NWAVES;
+                if (l < lt1 && l * TILE < maxlim) compute_tile<DT, E, EV, RB>(tr[i], qreg, lim, st, l * TILE, n, q, a.sc, kstage);
+                load_tile<DT, E, EV>(tr[i], kbase, vbase, (l + PF * NWAVES) * TILE, L, n, q, l + PF * NWAVES < lt1);
             }
         }
     }
 
+    HW_MARK(3);
     // ---- merge the four waves of the workgroup ----
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) st.l[rb] = quarter_sum(st.l[rb]);
@@ -443,9 +700,11 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     __syncthreads();
     if (wv == 1) put(0);
     __syncthreads();
+    HW_MARK(4);
 
     // ---- wave 0 stages the [row][ev] tile in LDS so that the global store is coalesced ----
-    float* stage = &x_lds[1][0][0];   // ROWS * EV floats <= NREG * 64
+    constexpr int SSTR = EV + 4;      // padded row stride: the 16 rows of a block land in different banks
+    float* stage = &x_lds[1][0][0];   // ROWS * SSTR floats == NREG * 64
     if (wv == 0) {
         add(0);
 #pragma unroll
@@ -453,7 +712,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) stage[(rb * 16 + n) * EV + out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
+                for (int i = 0; i < 4; ++i) stage[(rb * 16 + n) * SSTR + out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
             }
         }
         if (q == 0) {
@@ -461,7 +720,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
             for (int rb = 0; rb < RB; ++rb) {
                 const int r = r0 + rb * 16 + n;
                 if (r < a.R) {
-                    float* ml = a.part_ml + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r) * 2;
+                    HW_GLOBAL float* ml = a.part_ml + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r) * 2;
                     ml[0] = mall[rb];
                     ml[1] = st.l[rb];
                 }
@@ -471,33 +730,24 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     __syncthreads();
     {
         const int nrows = min(ROWS, a.R - r0);
-        float* dst = a.part_o + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r0) * EV;
-        for (int idx = tid * 4; idx < nrows * EV; idx += NTHREADS * 4)
-            *reinterpret_cast<f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + idx);
+        HW_GLOBAL float* dst = a.part_o + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r0) * EV;
+        for (int idx = tid * 4; idx < nrows * EV; idx += NTHREADS * 4) {
+            const int rr = idx / EV, e = idx - rr * EV;
+            *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * SSTR + e);
+        }
     }
 
+    HW_MARK(5);
     // rotated queries of zero-length fragments are still part of the operator's visible output
     if (a.rq != nullptr && g == 0 && !a.prerotated) {
-        for (int f = 0; f < a.F; ++f) {
-            if (a.frag.len[f] != 0) continue;
-            for (int idx = tid; idx < ROWS * E; idx += NTHREADS) {
-                const int rr = idx / E, e = idx - rr * E;
-                const int r = r0 + rr;
-                if (r >= a.R) continue;
-                const int ws = r / GQ, gq = r - ws * GQ;
-                const int w = ws / a.S, s = ws - w * a.S;
-                const size_t qrow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
-                const store_t* qp = reinterpret_cast<const store_t*>(a.q) + qrow * E;
-                const float x = Elem<DT>::to_float(qp[e]);
-                const int h = a.RotE >> 1;
-                float val = x;
-                if (e < a.RotE) {
-                    const size_t cs = ((size_t)(f * a.W + w) * a.S + s) * a.RotE;
-                    if (e < h) val = x * a.cos[cs + e] - Elem<DT>::to_float(qp[e + h]) * a.sin[cs + e];
-                    else val = x * a.cos[cs + e - h] + Elem<DT>::to_float(qp[e - h]) * a.sin[cs + e - h];
-                }
-                reinterpret_cast<store_t*>(a.rq)[((size_t)f * a.W * a.Hq * a.S + qrow) * E + e] = Elem<DT>::from_float(val);
-            }
+        unsigned long long empty = __ballot(lane < a.F && my_len == 0);
+        while (empty != 0) {
+            const int f = __builtin_ctzll(empty);
+            empty &= empty - 1;
+            __syncthreads();
+            QueryRotation<DT, E, ROWS, G::QSTR> qrot;
+            qrot.load(a, f, hkv, r0, GQ, tid);
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
         }
     }
 }
@@ -509,6 +759,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     constexpr int V4 = EV / 4;          // threads along the head dim (4 floats each)
     constexpr int NPG = 256 / V4;       // partial groups
     __shared__ __attribute__((aligned(16))) float red[NPG][EV];
+    __shared__ float wgt_lds[MAX_SPLITS];
+    __shared__ float red_m[4], red_l[4];
 
     const int hkv = blockIdx.x / a.R;
     const int r = blockIdx.x - hkv * a.R;
@@ -518,18 +770,55 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     const float* ml = a.part_ml + ((size_t)hkv * ns * a.R + r) * 2;
     const size_t mstride = (size_t)a.R * 2;
 
+    // one (max, sum) pair per thread, block-wide max and rescaled sum
+    float m_own[MAX_SPLITS / 256], l_own[MAX_SPLITS / 256];
     float M = NEG_BIG;
-    for (int s = 0; s < ns; ++s) M = fmaxf(M, ml[s * mstride]);
+#pragma unroll
+    for (int k = 0; k < MAX_SPLITS / 256; ++k) {
+        const int s = tid + k * 256;
+        m_own[k] = NEG_BIG;
+        l_own[k] = 0.f;
+        if (s < ns) {
+            const f32x2 v = *reinterpret_cast<const f32x2*>(ml + s * mstride);
+            m_own[k] = v.x;
+            l_own[k] = v.y;
+        }
+        M = fmaxf(M, m_own[k]);
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+    if ((tid & 63) == 0) red_m[tid >> 6] = M;
+    __syncthreads();
+    M = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
     float Lsum = 0.f;
-    for (int s = 0; s < ns; ++s) Lsum += ml[s * mstride + 1] * fast_exp2(ml[s * mstride] - M);
+#pragma unroll
+    for (int k = 0; k < MAX_SPLITS / 256; ++k) {
+        const int s = tid + k * 256;
+        const float wgt = fast_exp2(m_own[k] - M);
+        if (s < ns) wgt_lds[s] = wgt;
+        Lsum += l_own[k] * wgt;
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) Lsum += __shfl_xor(Lsum, off, 64);
+    if ((tid & 63) == 0) red_l[tid >> 6] = Lsum;
+    __syncthreads();
+    Lsum = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
 
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     const float* po = a.part_o + ((size_t)hkv * ns * a.R + r) * EV + e4 * 4;
-    for (int s = pg; s < ns; s += NPG) {
-        const float wgt = fast_exp2(ml[s * mstride] - M);
-        const f32x4 o = *reinterpret_cast<const f32x4*>(po + (size_t)s * a.R * EV);
-        acc += o * wgt;
+    const size_t ostride = (size_t)a.R * EV;
+    int s = pg;
+    for (; s + 3 * NPG < ns; s += 4 * NPG) {
+        const f32x4 o0 = *reinterpret_cast<const f32x4*>(po + (size_t)s * ostride);
+        const f32x4 o1 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + NPG) * ostride);
+        const f32x4 o2 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + 2 * NPG) * ostride);
+        const f32x4 o3 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + 3 * NPG) * ostride);
+        acc += o0 * wgt_lds[s];
+        acc += o1 * wgt_lds[s + NPG];
+        acc += o2 * wgt_lds[s + 2 * NPG];
+        acc += o3 * wgt_lds[s + 3 * NPG];
     }
+    for (; s < ns; s += NPG) acc += *reinterpret_cast<const f32x4*>(po + (size_t)s * ostride) * wgt_lds[s];
     *reinterpret_cast<f32x4*>(&red[pg][e4 * 4]) = acc;
     __syncthreads();
     if (pg == 0) {
@@ -537,8 +826,8 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
         const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
         const int GQ = a.Hq / a.Hkv;
         const int ws = r / GQ, gq = r - ws * GQ;
-        const int w = ws / a.S, s = ws - w * a.S;
-        const size_t orow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
+        const int w = ws / a.S, sq = ws - w * a.S;
+        const size_t orow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + sq);
         store_t* op = reinterpret_cast<store_t*>(a.out) + orow * EV + e4 * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i) op[i] = Elem<DT>::from_float(acc[i] * inv);
@@ -596,11 +885,11 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(u32x4* dst, const u32x
 // ------------------------------------------------------------------------------------------------
 template <class DT, int E, int EV>
 static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t stream) {
-    constexpr int W1 = Elem<DT>::size == 2 ? 2 : 1;
+    constexpr bool half = Elem<DT>::size == 2;
     if (rb == 1)
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, W1>), dim3(ka.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
     else
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1>), dim3(ka.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1, half ? 2 : 1>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
     return hipGetLastError();
 }
 
@@ -662,3 +951,9 @@ hipError_t launch_stream_copy(void* dst, const void* src, size_t bytes, hipStrea
 }
 
 }  // namespace hw
+
+#ifdef HW_CLOCKS
+extern "C" int hw_debug_read_clocks(unsigned long long* host, size_t n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(hw::hw_clock_buf), n * sizeof(unsigned long long));
+}
+#endif
