@@ -60,6 +60,8 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   len        HOST array of F lengths (the reference reads the same numbers from the tensor sizes, src/binding.cu:91)
  *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
+ *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
+ *              spread over more workgroups that read the same KV)
  *   ev_start / ev_stop   optional hipEvent_t recorded on `stream` immediately before / after the attention
  *                        kernel (not the merge kernel); pass NULL outside of profiling
  */
@@ -80,6 +82,7 @@ typedef struct hw_problem {
     void* workspace;
     size_t workspace_bytes;
     int32_t splits;
+    int32_t row_blocks;
     void* ev_start;
     void* ev_stop;
 } hw_problem;

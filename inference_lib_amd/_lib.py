@@ -38,7 +38,7 @@ class HwProblem(C.Structure):
         ("q", C.c_void_p), ("locations", C.c_void_p), ("cosines", C.c_void_p), ("sines", C.c_void_p),
         ("k", C.POINTER(C.c_void_p)), ("v", C.POINTER(C.c_void_p)), ("len", C.POINTER(C.c_int32)),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
-        ("splits", C.c_int32),
+        ("splits", C.c_int32), ("row_blocks", C.c_int32),
         ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p),
     ]
 
@@ -115,7 +115,7 @@ class Problem:
                  values: Sequence[torch.Tensor], scale: float, out: torch.Tensor,
                  cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
                  rq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                 prerotated: bool = False, splits: int = 0):
+                 prerotated: bool = False, splits: int = 0, row_blocks: int = 0):
         keys = [_frag3(k) for k in keys]
         values = [_frag3(v) for v in values]
         F = len(keys)
@@ -185,6 +185,7 @@ class Problem:
         p.v = C.cast(self._v, C.POINTER(C.c_void_p))
         p.len = C.cast(self._len, C.POINTER(C.c_int32))
         p.splits = int(splits)
+        p.row_blocks = int(row_blocks)
         self.p = p
         self.prerotated = prerotated
         self._ws = None
@@ -215,7 +216,8 @@ class Problem:
             check(fn(C.byref(self.p), C.c_void_p(stream)), fn.__name__)
 
 
-def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num_cus: int, splits: int = 0) -> HwPlan:
+def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num_cus: int, splits: int = 0,
+         dtype: int = HW_BF16, row_blocks: int = 0) -> HwPlan:
     """Host-only split plan (no GPU needed)."""
     F = len(lens)
     arr = (C.c_int32 * max(F, 1))(*lens)
@@ -223,6 +225,8 @@ def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num
     p.F, p.W, p.S, p.Hq, p.Hkv, p.Ev, p.E = F, W, S, Hq, Hkv, Ev, Ev
     p.len = C.cast(arr, C.POINTER(C.c_int32))
     p.splits = splits
+    p.dtype = dtype
+    p.row_blocks = row_blocks
     out = HwPlan()
     check(lib.hw_plan_debug(C.byref(p), num_cus, C.byref(out)), "hw_plan_debug")
     return out

@@ -71,6 +71,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
     const int rows = p->W * p->S * (p->Hq / p->Hkv);
     plan->rows = rows;
     plan->row_blocks = rows <= 16 ? 1 : 2;
+    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
     const int rows_per_wg = 16 * plan->row_blocks;
     plan->row_groups = (rows + rows_per_wg - 1) / rows_per_wg;
     plan->tile_tokens = hw::TILE;
@@ -146,6 +147,10 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
     const size_t parts = (size_t)p->Hkv * wgs;
     plan->workspace_bytes = parts * rows * ((size_t)p->Ev + 2) * sizeof(float);
     plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
+    // the attention kernel rotates in its prologue only over the full head dimension; any other rotary width
+    // goes through the standalone rotation first, into the caller's rq buffer or, without one, into the workspace
+    if (p->RotE != p->E && p->RotE >= 0)
+        plan->workspace_bytes += ((size_t)p->F * p->W * p->Hq * p->S * p->E * elem_size(p->dtype) + 255) & ~(size_t)255;
     return HW_OK;
 }
 
@@ -161,6 +166,19 @@ int run(const hw_problem* p, void* stream_, int fused) {
     if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    const void* q_in = p->q;
+    bool prerotated = !fused;
+    if (fused && p->RotE != p->E) {
+        void* rqbuf = p->rq;
+        if (rqbuf == nullptr) {
+            const size_t rqbytes = ((size_t)p->F * p->W * p->Hq * p->S * p->E * elem_size(p->dtype) + 255) & ~(size_t)255;
+            rqbuf = reinterpret_cast<char*>(p->workspace) + (plan.workspace_bytes - rqbytes);
+        }
+        hipError_t er = hw::launch_rope(rqbuf, p->q, p->cosines, p->sines, p->dtype, p->F, p->W, p->Hq, p->S, p->E, p->RotE, stream);
+        if (er != hipSuccess) return (int)er;
+        q_in = rqbuf;
+        prerotated = true;
+    }
     hw::KernelArgs ka;
     std::memset(&ka, 0, sizeof(ka));
     for (int f = 0; f < p->F; ++f) {
@@ -170,22 +188,22 @@ int run(const hw_problem* p, void* stream_, int fused) {
     }
     for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
     for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];
-    ka.h.q = p->q;
+    ka.h.q = q_in;
     ka.h.loc = p->locations;
     ka.h.cos = p->cosines;
     ka.h.sin = p->sines;
-    ka.h.rq = fused ? p->rq : nullptr;
+    ka.h.rq = (fused && !prerotated) ? p->rq : nullptr;
     const size_t parts = (size_t)p->Hkv * plan.wgs_per_head;
     ka.h.part_o = reinterpret_cast<float*>(p->workspace);
     ka.h.part_ml = ka.h.part_o + parts * plan.rows * p->Ev;
     ka.h.F = p->F; ka.h.W = p->W; ka.h.Hq = p->Hq; ka.h.Hkv = p->Hkv; ka.h.S = p->S;
-    ka.h.RotE = fused ? p->RotE : 0;
+    ka.h.RotE = prerotated ? 0 : p->RotE;
     ka.h.R = plan.rows;
     ka.h.nrg = plan.row_groups;
     ka.h.wgs_per_head = plan.wgs_per_head;
     ka.h.tiles_per_head = plan.tiles_per_head;
     ka.h.nwg = plan.workgroups;
-    ka.h.prerotated = fused ? 0 : 1;
+    ka.h.prerotated = prerotated ? 1 : 0;
     ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
     ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
 

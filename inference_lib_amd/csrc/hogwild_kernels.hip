@@ -26,6 +26,11 @@
 
 namespace hw {
 
+// tile buffers per wave of the two-row-block 16-bit kernels (tuning knob)
+#ifndef HW_PF2
+#define HW_PF2 2
+#endif
+
 // Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
 #ifdef HW_CLOCKS
 __device__ unsigned long long hw_clock_buf[4096 * 8];
@@ -117,6 +122,7 @@ struct Geo {
     static constexpr int SZ = Elem<DT>::size;
     static constexpr int KJ = E * SZ / 64;               // 16-byte K operand chunks per lane per 16-token block
     static constexpr int KROW = E * SZ;                  // bytes of one K row
+    static constexpr int VROW = EV * SZ;                 // bytes of one V row
     static constexpr int CPR = KROW / 16;                // 16-byte chunks per K row
     static constexpr int KL = TILE * KROW / 1024;        // 1 KB wave-wide K loads per tile
     static constexpr int KSTAGE = TILE * KROW;           // bytes of the per-wave K staging area in LDS
@@ -127,50 +133,80 @@ struct Geo {
     static constexpr int QSTR = E * SZ + 16;             // LDS row stride of the rotated query (bytes)
 };
 
-// Raw K/V registers of one 32-token tile of one wave.
+// Registers of one 32-token tile of one wave: only V lives in registers, K goes straight from global memory
+// into the wave's LDS staging slot.
 template <class DT, int E, int EV>
 struct TileRegs {
     typedef Geo<DT, E, EV> G;
-    u32x4 k[G::KL];      // the tile's K rows as one contiguous stream: load i, lane l holds chunk i*64 + l
-    u32 v[8][G::VW];
+    u32 v[8][G::VW];     // V rows of the lane's 8 reduction slots, VW dwords of each
 };
 
-// K/V fragment pointers arrive as integers out of the fragment table; they are given the global address
-// space explicitly so that the tile loads are global_load (vmcnt only), not flat_load.
-typedef const __attribute__((address_space(1))) char* gptr_t;
+#define HW_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 
-template <class DT, int E, int EV>
-__device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, gptr_t kbase, gptr_t vbase, int t0, int L, int n, int q,
-                                          bool real) {
-    typedef Geo<DT, E, EV> G;
-    // A tile past the end of the segment is still "loaded" so that the number of loads in flight is the same
-    // on every path (the wait counts then stay exact instead of draining everything); all its lanes read the
-    // first 16 bytes of the fragment, which costs one cache line.
-    const int last = real ? L - 1 : 0;
-    if (!real) t0 = 0, n = 0, q = 0;
-    const int lane = q * 16 + n;
-    // K: consecutive lanes read consecutive 16-byte chunks, so each load covers 1 KB of contiguous rows
+// A fragment's K and V slices of one kv head as buffer resources: out-of-range rows read as zero, so tiles
+// need no address clamping, and a tile that does not exist costs no memory traffic at all.
+struct FragView {
+    __amdgpu_buffer_rsrc_t k, v;
+};
+constexpr unsigned OOB_OFFSET = 0xFFFF0000u;   // beyond any fragment (lengths are validated on the host)
+
+__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int krow, int vrow) {
+    FragView fv;
+    fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * L * krow), 0, L * krow, 0x00020000);
+    fv.v = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(vptr + (unsigned long long)hkv * L * vrow), 0, L * vrow, 0x00020000);
+    return fv;
+}
+
+// LDS position of 16-byte chunk c of tile row `row` in a K staging slot.  The xor key makes the operand read
+// (16 lanes = 16 different rows, same chunk) touch 16 different 16-byte bank groups.
+template <class G>
+__device__ __forceinline__ int kstage_offset(int row, int c) {
+    const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+    return row * G::KROW + ((c ^ key) << 4);
+}
+
+// Per-lane byte offsets (within a tile) of the K chunk each lane fetches in each of the KL wave-wide loads.
+// A load writes LDS linearly (lane l -> slot base + 16 l), so the bank swizzle of kstage_offset is applied on
+// the global side: the lane that fills position (row, slot) fetches chunk slot ^ key(row) of that row.  The 16
+// lanes of a row still cover the row's bytes exactly once, so every load remains 1 KB of whole rows.
+template <class G>
+__device__ __forceinline__ void k_lane_offsets(unsigned* koff, int lane) {
 #pragma unroll
     for (int i = 0; i < G::KL; ++i) {
-        const int g = real ? i * 64 + lane : 0;
-        const int tok = min(t0 + g / G::CPR, last);
-        t.k[i] = *reinterpret_cast<const __attribute__((address_space(1))) u32x4*>(kbase + (size_t)tok * G::KROW + (g % G::CPR) * 16);
+        const int p = i * 64 + lane;
+        const int row = p / G::CPR, slot = p % G::CPR;
+        const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+        koff[i] = row * G::KROW + ((slot ^ key) << 4);
     }
+}
+
+// Issue the loads of one tile: K by direct global->LDS transfers into `kslot` (this wave's part of a staging
+// slot), V into registers.  The number of load instructions is the same whether or not the tile exists, which
+// keeps the hardware wait counts exact on every path; a tile that does not exist reads out of range (zeros,
+// no memory traffic).
+template <class DT, int E, int EV>
+__device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView& fv, char* kslot, const unsigned* koff, int t0,
+                                          int n, int q, bool real) {
+    typedef Geo<DT, E, EV> G;
+    const unsigned kb = real ? (unsigned)(t0 * G::KROW) : OOB_OFFSET;
+#pragma unroll
+    for (int i = 0; i < G::KL; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, 0);
+    // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load
+    const unsigned vb = real ? (unsigned)((t0 + q * 4) * G::VROW + n * (G::VLD * 4)) : OOB_OFFSET;
 #pragma unroll
     for (int idx = 0; idx < 8; ++idx) {
-        int tok = min(t0 + slot_token(q, idx), last);
-        gptr_t row = vbase + (size_t)tok * (EV * G::SZ);
+        const int rowoff = ((idx >> 2) * 16 + (idx & 3)) * G::VROW;
 #pragma unroll
         for (int hh = 0; hh < G::NVL; ++hh) {
-            gptr_t p = row + hh * 256 + n * (G::VLD * 4);
             if constexpr (G::VLD == 4) {
-                u32x4 x = *reinterpret_cast<const __attribute__((address_space(1))) u32x4*>(p);
+                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(fv.v, vb + rowoff + hh * 256, 0, 0);
                 t.v[idx][hh * 4 + 0] = x.x;
                 t.v[idx][hh * 4 + 1] = x.y;
                 t.v[idx][hh * 4 + 2] = x.z;
                 t.v[idx][hh * 4 + 3] = x.w;
             } else {
-                u32x2 x = *reinterpret_cast<const __attribute__((address_space(1))) u32x2*>(p);
+                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(fv.v, vb + rowoff, 0, 0);
                 t.v[idx][0] = x.x;
                 t.v[idx][1] = x.y;
             }
@@ -178,86 +214,83 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, gptr_t kbase, 
     }
 }
 
-// LDS position of 16-byte chunk c of tile row `row` in the per-wave K staging area.  The xor key makes both
-// the coalesced write (16 consecutive lanes = consecutive chunks) and the operand read (16 lanes = 16
-// different rows, same chunk) touch 16 different 16-byte bank groups.
-template <class G>
-__device__ __forceinline__ int kstage_offset(int row, int c) {
-    const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
-    return row * G::KROW + ((c ^ key) << 4);
-}
-
 // Running state of one wave: RB row blocks of 16 rows each.
 template <int RB, int NOC>
 struct WaveState {
     f32x4 o[RB][NOC];
-    float m[RB];
+    float m[RB];   // running max of scale*log2(e)*q.k
     float l[RB];   // lane-partial sum: this lane's quarter of the tokens
 };
 
-template <class DT, int E, int EV, int RB>
-__device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const u32x4 (&qreg)[RB][Geo<DT, E, EV>::KJ],
-                                             const int (&lim)[RB], WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q,
-                                             float sc, char* kstage) {
+// One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG>
+__device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
+                                             WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage) {
     typedef Geo<DT, E, EV> G;
-    // K: registers (stream order) -> LDS -> registers in MFMA A-operand order (lane = token, 16 B of head dim).
-    // The staging area is private to the wave and LDS executes a wave's instructions in order.
+#ifdef HW_NO_COMPUTE   // tuning aid: consume the tile without doing the arithmetic
     {
-        const int lane = q * 16 + n;
+        u32 x = 0;
 #pragma unroll
-        for (int i = 0; i < G::KL; ++i) {
-            const int g = i * 64 + lane;
-            *reinterpret_cast<u32x4*>(kstage + kstage_offset<G>(g / G::CPR, g % G::CPR)) = t.k[i];
-        }
+        for (int idx = 0; idx < 8; ++idx)
+#pragma unroll
+            for (int d = 0; d < G::VW; ++d) x ^= t.v[idx][d];
+        x ^= *reinterpret_cast<const u32*>(kstage + kstage_offset<G>(n, q));
+        st.l[0] += __uint_as_float(x & 0x3fffffffu);
+        return;
     }
-    __builtin_amdgcn_wave_barrier();
-    u32x4 kop[2][G::KJ];
+#endif
+    // K operand: out of the staging slot in MFMA A-operand order (lane = token, 16 B of head dim).  The compiler
+    // tracks the outstanding global->LDS transfers per staging slot and waits for this slot's before the reads.
+    // S^T blocks: for each 16-token block, its K operand (lane = token, 16 B of head dim per k-step) against the
+    // B operand of every row block (this row's rotated query, from registers when QREG, else straight from LDS)
+    f32x4 sacc[RB][2];
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
+        u32x4 kop[G::KJ];
 #pragma unroll
-        for (int j = 0; j < G::KJ; ++j)
-            kop[tb][j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
-    }
-    __builtin_amdgcn_wave_barrier();
-    float p[RB][8];
+        for (int j = 0; j < G::KJ; ++j) kop[j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
 #pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        f32x4 sacc[2];
+        for (int rb = 0; rb < RB; ++rb) {
+            u32x4 qop[G::KJ];
 #pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
+            for (int j = 0; j < G::KJ; ++j)
+                qop[j] = QREG ? qreg[rb * G::KJ + j] : *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
             if constexpr (G::SZ == 2) {
 #pragma unroll
-                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[tb][j], qreg[rb][j], acc);
+                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[j], qop[j], acc);
             } else {
 #pragma unroll
                 for (int j = 0; j < G::KJ; ++j) {
 #pragma unroll
                     for (int c = 0; c < 4; ++c)
-                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(kop[tb][j][c]), __uint_as_float(qreg[rb][j][c]),
-                                                                   acc, 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(kop[j][c]), __uint_as_float(qop[j][c]), acc, 0, 0, 0);
                 }
             }
-            sacc[tb] = acc;
+            sacc[rb][tb] = acc;
         }
+    }
+    float p[RB][8];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
         float s[8];
-        bool ok[8];
         float mx = NEG_BIG;
 #pragma unroll
         for (int idx = 0; idx < 8; ++idx) {
-            s[idx] = sacc[idx >> 2][idx & 3] * sc;
-            ok[idx] = (t0 + slot_token(q, idx)) < lim[rb];
-            mx = ok[idx] ? fmaxf(mx, s[idx]) : mx;
+            s[idx] = sacc[rb][idx >> 2][idx & 3];
+            if constexpr (MASKED) s[idx] = (t0 + slot_token(q, idx)) < lim[rb] ? s[idx] : NEG_BIG;
+            mx = fmaxf(mx, s[idx]);
         }
-        mx = quarter_max(mx);
-        float mnew = fmaxf(st.m[rb], mx);
-        float alpha = fast_exp2(st.m[rb] - mnew);
+        mx = quarter_max(mx) * sc;                     // sc > 0: scaling commutes with the max
+        const float mnew = fmaxf(st.m[rb], mx);
+        const float alpha = fast_exp2(st.m[rb] - mnew);
         st.m[rb] = mnew;
+        // a row that has seen nothing yet has mnew ~ -1e29; exponentiate against 0 so its masked slots give 0, not 1
+        const float mref = MASKED ? (mnew < -1.0e28f ? 0.f : mnew) : mnew;
         float psum = 0.f;
 #pragma unroll
         for (int idx = 0; idx < 8; ++idx) {
-            float e = fast_exp2(s[idx] - mnew);
-            p[rb][idx] = ok[idx] ? e : 0.f;
+            p[rb][idx] = fast_exp2(__builtin_fmaf(s[idx], sc, -mref));
             psum += p[rb][idx];
         }
         st.l[rb] = st.l[rb] * alpha + psum;
@@ -391,114 +424,79 @@ __device__ __forceinline__ RowMap map_row(const DevHeader& a, int r, int hkv, in
 
 // Query rotation of one fragment, split in two phases so that its few global loads can be issued BEFORE the
 // K/V tile loads (loads return in issue order, so a dependent wait would otherwise drain the whole KV
-// prefetch first) and consumed after them.  One work item = one 16-byte chunk pair (e, e + RotE/2) of one
-// row, or one pass-through chunk.  Index convention of src/rope.cuh:18-51: both halves read cos/sin at the
-// first-half index.  Rotary widths that are not a multiple of two chunks take the scalar path in phase two.
-template <class DT, int E, int ROWS, int QSTR>
+// prefetch first) and consumed after them.  The kernel rotates over the full head dimension only (RotE == E,
+// what the models on this path use); other rotary widths are rotated by the standalone kernel first and
+// enter here as pre-rotated queries.  One work item = one 16-byte chunk pair (e, e + E/2) of one row; the
+// item count per thread is a compile-time constant.  Index convention of src/rope.cuh:18-51: both halves
+// read cos/sin at the first-half index.
+// PRE = the queries arrive already rotated, [F,W,Hq,S,E] (the hogwild_sdpa entry): one item = one chunk copy.
+template <class DT, int E, int ROWS, int QSTR, bool PRE>
 struct QueryRotation {
-    typedef typename Elem<DT>::store_t store_t;
     static constexpr int SZ = Elem<DT>::size;
     static constexpr int CH = Chunk<DT>::CH;
-    static constexpr int NIT = (ROWS * (E / CH) + NTHREADS - 1) / NTHREADS;   // items per thread, worst case (no rotation)
+    static constexpr int IPR = PRE ? E / CH : E / (2 * CH);                  // items per row
+    static constexpr int NIT = (ROWS * IPR + NTHREADS - 1) / NTHREADS;       // items per thread
 
-    u32x4 xa[NIT], xb[NIT];
-    f32x4 cs[NIT][CH / 4], sn[NIT][CH / 4];
-
-    static __device__ __forceinline__ bool vec_ok(int rot) { return (rot % (2 * CH)) == 0; }
+    u32x4 xa[NIT];
+    u32x4 xb[PRE ? 1 : NIT];
+    f32x4 cs[PRE ? 1 : NIT][CH / 4], sn[PRE ? 1 : NIT][CH / 4];
 
     __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid) {
-        const int rot = a.prerotated ? 0 : a.RotE;
-        if (!vec_ok(rot)) return;
         const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
-        const int npair = (rot / 2) / CH;
-        const int ipr = npair + (E - rot) / CH;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
             const int item = tid + it * NTHREADS;
-            const int rr = item / ipr, slot = item - rr * ipr;
-            const int r = r0 + rr;
-            if (item >= ROWS * ipr || r >= a.R) continue;
+            const int rr = item / IPR, slot = item % IPR;
+            // rows beyond R (MFMA padding) and threads beyond the item count read row 0: harmless, and keeps the
+            // loads out of divergent control flow
+            const int r = (item < ROWS * IPR && r0 + rr < a.R) ? r0 + rr : r0;
             const RowMap rm = map_row(a, r, hkv, GQ);
-            const HW_GLOBAL char* qp = a.q + (rm.qrow * E + (a.prerotated ? f * fstride : 0)) * SZ;
-            if (slot < npair) {
-                xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
-                xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + npair) * 16);
-                const size_t co = ((size_t)f * a.W * a.S + rm.ws) * a.RotE + slot * CH;
+            const HW_GLOBAL char* qp = a.q + (rm.qrow * E + (PRE ? f * fstride : 0)) * SZ;
+            xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
+            if constexpr (!PRE) {
+                xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + IPR) * 16);
+                const size_t co = ((size_t)f * a.W * a.S + rm.ws) * E + slot * CH;
 #pragma unroll
                 for (int i = 0; i < CH / 4; ++i) {
                     cs[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.cos + co + 4 * i);
                     sn[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.sin + co + 4 * i);
                 }
-            } else {
-                xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + npair) * 16);
             }
         }
     }
 
     __device__ __forceinline__ void finish(const DevHeader& a, char* q_lds, int f, int hkv, int r0, int GQ, bool write_rq,
                                            int tid) const {
-        const int rot = a.prerotated ? 0 : a.RotE;
         const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
-        if (vec_ok(rot)) {
-            const int npair = (rot / 2) / CH;
-            const int ipr = npair + (E - rot) / CH;
 #pragma unroll
-            for (int it = 0; it < NIT; ++it) {
-                const int item = tid + it * NTHREADS;
-                const int rr = item / ipr, slot = item - rr * ipr;
-                const int r = r0 + rr;
-                if (item >= ROWS * ipr) continue;
-                char* lrow = q_lds + rr * QSTR;
-                if (r >= a.R) {   // padding rows of the 16-row MFMA block
-                    const u32x4 z = {0, 0, 0, 0};
-                    if (slot < npair) *reinterpret_cast<u32x4*>(lrow + slot * 16) = z;
-                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = z;
-                    continue;
-                }
-                const RowMap rm = map_row(a, r, hkv, GQ);
-                HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
-                if (slot < npair) {
-                    float x1[CH], x2[CH], y1[CH], y2[CH];
-                    Chunk<DT>::unpack(xa[it], x1);
-                    Chunk<DT>::unpack(xb[it], x2);
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / IPR, slot = item % IPR;
+            if (item >= ROWS * IPR) continue;
+            char* lrow = q_lds + rr * QSTR;
+            const bool pad = r0 + rr >= a.R;   // padding rows of the 16-row MFMA block hold zeros
+            const u32x4 z = {0, 0, 0, 0};
+            if constexpr (PRE) {
+                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : xa[it];
+            } else {
+                float x1[CH], x2[CH], y1[CH], y2[CH];
+                Chunk<DT>::unpack(xa[it], x1);
+                Chunk<DT>::unpack(xb[it], x2);
 #pragma unroll
-                    for (int i = 0; i < CH; ++i) {
-                        const float c = cs[it][i >> 2][i & 3], sv = sn[it][i >> 2][i & 3];
-                        y1[i] = x1[i] * c - x2[i] * sv;
-                        y2[i] = x2[i] * c + x1[i] * sv;
-                    }
-                    const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
-                    *reinterpret_cast<u32x4*>(lrow + slot * 16) = ya;
-                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = yb;
-                    if (write_rq) {
-                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
-                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + npair) * 16) = yb;
-                    }
-                } else {
-                    *reinterpret_cast<u32x4*>(lrow + (slot + npair) * 16) = xa[it];
-                    if (write_rq) *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + npair) * 16) = xa[it];
+                for (int i = 0; i < CH; ++i) {
+                    const float c = cs[it][i >> 2][i & 3], sv = sn[it][i >> 2][i & 3];
+                    y1[i] = x1[i] * c - x2[i] * sv;
+                    y2[i] = x2[i] * c + x1[i] * sv;
                 }
-            }
-        } else {
-            const int h = rot >> 1;
-            for (int idx = tid; idx < ROWS * E; idx += NTHREADS) {
-                const int rr = idx / E, e = idx - rr * E;
-                const int r = r0 + rr;
-                store_t sv = Elem<DT>::from_float(0.f);
-                if (r < a.R) {
-                    const RowMap rm = map_row(a, r, hkv, GQ);
-                    const HW_GLOBAL store_t* qp = reinterpret_cast<const HW_GLOBAL store_t*>(a.q) + rm.qrow * E;
-                    const float x = Elem<DT>::to_float(qp[e]);
-                    float val = x;
-                    if (e < rot) {
-                        const size_t co = ((size_t)f * a.W * a.S + rm.ws) * a.RotE;
-                        if (e < h) val = x * a.cos[co + e] - Elem<DT>::to_float(qp[e + h]) * a.sin[co + e];
-                        else val = x * a.cos[co + e - h] + Elem<DT>::to_float(qp[e - h]) * a.sin[co + e - h];
-                    }
-                    sv = Elem<DT>::from_float(val);
-                    if (write_rq) reinterpret_cast<HW_GLOBAL store_t*>(a.rq)[(f * fstride + rm.qrow * E) + e] = sv;
+                const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
+                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : ya;
+                *reinterpret_cast<u32x4*>(lrow + (slot + IPR) * 16) = pad ? z : yb;
+                if (write_rq && !pad) {
+                    const RowMap rm = map_row(a, r0 + rr, hkv, GQ);
+                    HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
+                    *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
+                    *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + IPR) * 16) = yb;
                 }
-                *reinterpret_cast<store_t*>(q_lds + rr * QSTR + e * SZ) = sv;
             }
         }
     }
@@ -506,34 +504,45 @@ struct QueryRotation {
 
 // MINW = waves per SIMD the register budget is sized for: 2 (<= 256 VGPRs) when one 16-row block is live,
 // 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the tile registers too large.
-// PF = tiles a wave keeps in flight.
-template <class DT, int E, int EV, int RB, int MINW, int PF>
+// PF = tiles a wave keeps in flight.  PRE = queries arrive rotated (hogwild_sdpa), else fused rotation.
+template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE>
 __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
-    typedef typename Elem<DT>::store_t store_t;
     constexpr int ROWS = RB * 16;
-    constexpr int NREG = RB * G::NOC * 4 + RB;  // accumulator floats + l per lane exchanged between waves
+    constexpr int SSTR = EV + 4;      // padded row stride of the epilogue exchange: rows land in different banks
 
+    struct Exchange {                 // what each wave hands over at the end
+        float o[NWAVES][ROWS][SSTR];
+        float m[NWAVES][ROWS];
+        float l[NWAVES][ROWS];
+    };
+    constexpr int SBYTES = NWAVES * G::KSTAGE;
     __shared__ __attribute__((aligned(16))) char q_lds[ROWS * G::QSTR];
     __shared__ int lim_lds[ROWS];
-    __shared__ float m_lds[NWAVES][ROWS];
-    // wave-exchange buffers of the epilogue, aliased with the per-wave K staging areas of the main loop
-    constexpr int XBYTES = 2 * NREG * 64 * 4;
-    constexpr int SBYTES = NWAVES * G::KSTAGE;
-    __shared__ __attribute__((aligned(16))) char xs_lds[XBYTES > SBYTES ? XBYTES : SBYTES];
-    float (*x_lds)[NREG][64] = reinterpret_cast<float (*)[NREG][64]>(xs_lds);
+    // One K staging slot per tile in flight, each a separate LDS object so that the wait for a slot's incoming
+    // transfers does not extend to the other slots.  The epilogue exchange reuses the memory of slot 0.
+    union Slot0 {
+        char k[SBYTES];
+        Exchange ex;
+    };
+    __shared__ __attribute__((aligned(16))) Slot0 slot0;
+    __shared__ __attribute__((aligned(16))) char slot1[PF > 1 ? SBYTES : 16];
+    __shared__ __attribute__((aligned(16))) char slot2[PF > 2 ? SBYTES : 16];
+    static_assert(PF <= 3, "three staging slots");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int q = lane >> 4;
-    char* kstage = xs_lds + wv * G::KSTAGE;
+    char* const kslots[3] = {slot0.k + wv * G::KSTAGE, slot1 + (PF > 1 ? wv * G::KSTAGE : 0), slot2 + (PF > 2 ? wv * G::KSTAGE : 0)};
+    unsigned koff[G::KL];
+    k_lane_offsets<G>(koff, lane);
 
     // Everything the kernel needs from its arguments is requested here in one burst, before anything waits:
-    // the 32 scalar dwords with two 64-byte scalar loads, the fragment table and the workgroup boundary table
-    // with one vector load per lane and array.  The argument segment is slow to reach and the compiler would
-    // otherwise fetch it lazily, one dependent round trip after another.
+    // the fragment table and the workgroup boundary table with one vector load per lane and array, the 32
+    // scalar dwords with two 64-byte scalar loads.  The argument segment is slow to reach and the compiler
+    // would otherwise fetch it lazily, one dependent round trip after another.
     const int fl = lane & (MAXF - 1);
     const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
     const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
@@ -599,153 +608,135 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
                                       (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
         const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
                                       (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
-        gptr_t kbase = (gptr_t)(kp + (unsigned long long)hkv * L * (E * G::SZ));
-        gptr_t vbase = (gptr_t)(vp + (unsigned long long)hkv * L * (EV * G::SZ));
+        const FragView fv = make_view(kp, vp, hkv, L, G::KROW, G::VROW);
         const int lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
         const int lt1 = s1 - fb;
 
         // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first PF
         // K/V tiles; the rotation then waits only for the former while the tiles stay in flight
-        QueryRotation<DT, E, ROWS, G::QSTR> qrot;
+        QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
         qrot.load(a, f, hkv, r0, GQ, tid);
         // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
         const int lm = a.loc[(size_t)f * a.W * a.S + min(r0 + (tid & (ROWS - 1)), a.R - 1) / GQ];
+        // the first tile is requested before the prologue, further look-ahead tiles after it: a wave stalls
+        // while the memory pipeline accepts its requests, and the prologue should not sit behind that stall
         TileRegs<DT, E, EV> tr[PF];
-#pragma unroll
-        for (int i = 0; i < PF; ++i)
-            load_tile<DT, E, EV>(tr[i], kbase, vbase, (lt0 + i * NWAVES) * TILE, L, n, q, lt0 + i * NWAVES < lt1);
+        if (PF > 1) load_tile<DT, E, EV>(tr[0], fv, kslots[0], koff, lt0 * TILE, n, q, lt0 < lt1);
 
         HW_MARK(1);
         // ---- prologue: rotate the queries of this fragment into LDS ----
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
         qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && s0 == fb, tid);
-        if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0;
+        // rows that pad the MFMA block get "sees everything": their query is zero and they are never stored,
+        // and they must not keep the unmasked fast path from being taken
+        if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
         __syncthreads();
 
-        u32x4 qreg[RB][G::KJ];
+        // with one wave per SIMD there are registers to spare: keep the query operands of the segment in them
+        constexpr bool QREG = MINW == 1;
+        u32x4 qreg[QREG ? RB * G::KJ : 1];
+        if constexpr (QREG) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                for (int j = 0; j < G::KJ; ++j)
+                    qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+        }
         int lim[RB];
-        int maxlim = 0;
+        int maxlim = 0, minlim = 0x7fffffff;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-            for (int j = 0; j < G::KJ; ++j)
-                qreg[rb][j] = *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
             lim[rb] = lim_lds[rb * 16 + n];
-            maxlim = max(maxlim, lim[rb]);
+            const bool pad = r0 + rb * 16 + n >= a.R;
+            maxlim = max(maxlim, pad ? 0 : lim[rb]);
+            minlim = min(minlim, lim[rb]);
         }
 #pragma unroll
-        for (int off = 1; off < 16; off <<= 1) maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
+        for (int off = 1; off < 16; off <<= 1) {
+            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
+            minlim = min(minlim, __shfl_xor(minlim, off, 64));
+        }
         maxlim = __builtin_amdgcn_readfirstlane(maxlim);
+        minlim = __builtin_amdgcn_readfirstlane(minlim);
         HW_MARK(2);
+#pragma unroll
+        for (int i = 1; i < PF - 1; ++i)
+            load_tile<DT, E, EV>(tr[i], fv, kslots[i], koff, (lt0 + i * NWAVES) * TILE, n, q, lt0 + i * NWAVES < lt1);
 
-        // ---- stream this wave's tiles, PF in flight ----
+        // ---- stream this wave's tiles: PF buffers, the tile PF-1 steps ahead is requested right before each
+        // tile is computed, so its transfer overlaps the arithmetic and the prologue above overlapped the first ----
         for (int lt = lt0; lt < lt1; lt += PF * NWAVES) {
 #pragma unroll
             for (int i = 0; i < PF; ++i) {
                 const int l = lt + i * NWAVES;
-                if (l < lt1 && l * TILE < maxlim) compute_tile<DT, E, EV, RB>(tr[i], qreg, lim, st, l * TILE, n, q, a.sc, kstage);
-                load_tile<DT, E, EV>(tr[i], kbase, vbase, (l + PF * NWAVES) * TILE, L, n, q, l + PF * NWAVES < lt1);
+                const int t0 = l * TILE;
+                const int nb = (i + PF - 1) % PF;   // constant after unrolling
+                const int ln = l + (PF - 1) * NWAVES;
+                load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
+                if (l < lt1 && t0 < maxlim) {
+                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                    else compute_tile<DT, E, EV, RB, true, QREG>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                }
             }
         }
     }
 
     HW_MARK(3);
-    // ---- merge the four waves of the workgroup ----
+    // ---- merge the four waves of the workgroup: every wave hands over its raw accumulators, running max and
+    // sum; then all threads combine them with the weights 2^(m_wave - m_max) and store coalesced ----
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) st.l[rb] = quarter_sum(st.l[rb]);
-    __syncthreads();
-    if (q == 0) {
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) m_lds[wv][rb * 16 + n] = st.m[rb];
-    }
-    __syncthreads();
-    float mall[RB];
+    __syncthreads();   // every wave is done with K staging slot 0, whose memory the exchange buffer reuses
+    Exchange& ex = slot0.ex;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-        float mm = m_lds[0][rb * 16 + n];
 #pragma unroll
-        for (int w2 = 1; w2 < NWAVES; ++w2) mm = fmaxf(mm, m_lds[w2][rb * 16 + n]);
-        mall[rb] = mm;
-        const float fsc = fast_exp2(st.m[rb] - mm);
-        st.l[rb] *= fsc;
+        for (int c = 0; c < G::NOC; ++c) {
 #pragma unroll
-        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] *= fsc;
-    }
-    // tree sum over waves: (2,3) -> (0,1), then 1 -> 0.  Deterministic order.
-    auto put = [&](int slot) {
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-            for (int c = 0; c < G::NOC; ++c) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) x_lds[slot][(rb * G::NOC + c) * 4 + i][lane] = st.o[rb][c][i];
-            }
-            x_lds[slot][RB * G::NOC * 4 + rb][lane] = st.l[rb];
-        }
-    };
-    auto add = [&](int slot) {
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-            for (int c = 0; c < G::NOC; ++c) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) st.o[rb][c][i] += x_lds[slot][(rb * G::NOC + c) * 4 + i][lane];
-            }
-            st.l[rb] += x_lds[slot][RB * G::NOC * 4 + rb][lane];
-        }
-    };
-    if (wv >= 2) put(wv - 2);
-    __syncthreads();
-    if (wv < 2) add(wv);
-    __syncthreads();
-    if (wv == 1) put(0);
-    __syncthreads();
-    HW_MARK(4);
-
-    // ---- wave 0 stages the [row][ev] tile in LDS so that the global store is coalesced ----
-    constexpr int SSTR = EV + 4;      // padded row stride: the 16 rows of a block land in different banks
-    float* stage = &x_lds[1][0][0];   // ROWS * SSTR floats == NREG * 64
-    if (wv == 0) {
-        add(0);
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-#pragma unroll
-            for (int c = 0; c < G::NOC; ++c) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) stage[(rb * 16 + n) * SSTR + out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
-            }
+            for (int i = 0; i < 4; ++i) ex.o[wv][rb * 16 + n][out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
         }
         if (q == 0) {
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                const int r = r0 + rb * 16 + n;
-                if (r < a.R) {
-                    HW_GLOBAL float* ml = a.part_ml + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r) * 2;
-                    ml[0] = mall[rb];
-                    ml[1] = st.l[rb];
-                }
-            }
+            ex.m[wv][rb * 16 + n] = st.m[rb];
+            ex.l[wv][rb * 16 + n] = st.l[rb];
         }
     }
     __syncthreads();
+    HW_MARK(4);
     {
         const int nrows = min(ROWS, a.R - r0);
-        HW_GLOBAL float* dst = a.part_o + ((size_t)(hkv * a.wgs_per_head + g) * a.R + r0) * EV;
+        const size_t part = (size_t)(hkv * a.wgs_per_head + g) * a.R + r0;
+        HW_GLOBAL float* dst = a.part_o + part * EV;
         for (int idx = tid * 4; idx < nrows * EV; idx += NTHREADS * 4) {
             const int rr = idx / EV, e = idx - rr * EV;
-            *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * SSTR + e);
+            float mm = ex.m[0][rr];
+#pragma unroll
+            for (int w2 = 1; w2 < NWAVES; ++w2) mm = fmaxf(mm, ex.m[w2][rr]);
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            float lsum = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < NWAVES; ++w2) {
+                const float wgt = fast_exp2(ex.m[w2][rr] - mm);
+                acc += *reinterpret_cast<const f32x4*>(&ex.o[w2][rr][e]) * wgt;
+                lsum += ex.l[w2][rr] * wgt;
+            }
+            *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = acc;
+            if (e == 0) {
+                HW_GLOBAL float* ml = a.part_ml + (part + rr) * 2;
+                ml[0] = mm;
+                ml[1] = lsum;
+            }
         }
     }
-
     HW_MARK(5);
+
     // rotated queries of zero-length fragments are still part of the operator's visible output
-    if (a.rq != nullptr && g == 0 && !a.prerotated) {
+    if (!PRE && a.rq != nullptr && g == 0) {
         unsigned long long empty = __ballot(lane < a.F && my_len == 0);
         while (empty != 0) {
             const int f = __builtin_ctzll(empty);
             empty &= empty - 1;
             __syncthreads();
-            QueryRotation<DT, E, ROWS, G::QSTR> qrot;
+            QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
             qrot.load(a, f, hkv, r0, GQ, tid);
             qrot.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
         }
@@ -883,20 +874,25 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(u32x4* dst, const u32x
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-template <class DT, int E, int EV>
+template <class DT, int E, int EV, bool PRE>
 static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t stream) {
     constexpr bool half = Elem<DT>::size == 2;
     if (rb == 1)
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
+                           stream, ka);
     else
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1, half ? 2 : 1>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1, half ? HW_PF2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
     return hipGetLastError();
 }
 
 template <class DT>
 static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, hipStream_t stream) {
-    if (E == 128) return launch_attention_rb<DT, 128, 128>(ka, rb, stream);
-    return launch_attention_rb<DT, 64, 64>(ka, rb, stream);
+    if (ka.h.prerotated) {
+        if (E == 128) return launch_attention_rb<DT, 128, 128, true>(ka, rb, stream);
+        return launch_attention_rb<DT, 64, 64, true>(ka, rb, stream);
+    }
+    if (E == 128) return launch_attention_rb<DT, 128, 128, false>(ka, rb, stream);
+    return launch_attention_rb<DT, 64, 64, false>(ka, rb, stream);
 }
 
 hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream) {

@@ -38,3 +38,48 @@ def test_baseline_configs(oracle, idx):
     e1 = assert_close("out", out, o_ref, TOL[c.dtype])
     e2 = assert_close("lse", lse, l_ref, TOL[c.dtype])
     print(f"  max err out {e1:.3e} lse {e2:.3e}", flush=True)
+
+
+@pytest.mark.parametrize("dtype,E", [("bf16", 128), ("f16", 64), ("f32", 64), ("f32", 128)])
+def test_rope_and_sdpa_entries(oracle, dtype, E):
+    """hw_rope and hw_sdpa (pre-rotated queries), the two halves the reference also exports separately
+    (python/hogwild/attention.py:26-35, 70-74)."""
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype=dtype, W=3, S=2, Hq=6, Hkv=2, E=E, lens=(70, 33, 1, 64), seed=5)
+    cd = c.to(_dev())
+    print(f"case {c.name} E={E}", flush=True)
+    W, Hq, S, _ = cd.q.shape
+    rq = torch.full((c.F, W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    _lib.rope(cd.q, cd.cos, cd.sin, rq)
+    torch.cuda.synchronize()
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("rope", rq, rq_ref, 1e-5 if dtype == "f32" else 3.2e-2)
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    pr = _lib.Problem(q=rq, locations=cd.locations, keys=cd.keys, values=cd.values, scale=c.scale, out=out, lse=lse,
+                      prerotated=True)
+    pr.run()
+    torch.cuda.synchronize()
+    # the oracle attends with the GPU's own rotated queries so this checks the attention half alone
+    o2, l2 = oracle.sdpa_fragments(np64(rq), c.locations.numpy(), [np64(k) for k in c.keys], [np64(v) for v in c.values], c.scale)
+    assert_close("sdpa out", out, o2, TOL[dtype])
+    assert_close("sdpa lse", lse, l2, TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype,E,rot", [("bf16", 128, 64), ("f16", 64, 32), ("f32", 64, 20), ("bf16", 128, 0)])
+def test_partial_rotary(oracle, dtype, E, rot):
+    """Rotary width smaller than the head dim (pass-through tail, src/rope.cuh:48-51), including widths that
+    are not a multiple of the 16-byte vector width and no rotation at all."""
+    from inference_lib_amd import cases
+    c = cases.small_case(dtype=dtype, W=2, S=2, Hq=4, Hkv=2, E=E, lens=(90, 40, 47), seed=21, rot_dim=max(rot, 2))
+    if rot == 0:   # zero-width tables: nothing is rotated
+        c.cos = c.cos[..., :0].contiguous()
+        c.sin = c.sin[..., :0].contiguous()
+    print(f"case {c.name} E={E} rot={rot}", flush=True)
+    out, lse, rq = run_fused(c.to(_dev()))
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("rq", rq, rq_ref, 1e-5 if dtype == "f32" else 3.2e-2)
+    assert_close("out", out, o_ref, TOL[dtype])
+    assert_close("lse", lse, l_ref, TOL[dtype])
+    out2, lse2, _ = run_fused(c.to(_dev()), with_rq=False)     # rotated queries go to the workspace instead
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
