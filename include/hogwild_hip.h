@@ -34,7 +34,8 @@ typedef enum hw_status {
     HW_OK = 0,
     HW_ERR_NULL = -1,          /* a required pointer is NULL */
     HW_ERR_DTYPE = -2,         /* dtype is not one of hw_dtype */
-    HW_ERR_SHAPE = -3,         /* a dimension is non-positive or inconsistent (Hq % Hkv, RotE > E, odd RotE, ...) */
+    HW_ERR_SHAPE = -3,         /* a dimension is non-positive or inconsistent (Hq % Hkv, RotE > E, odd RotE, a fragment
+                                  whose kv-head slice reaches 2 GiB, scale not positive and finite, ...) */
     HW_ERR_UNSUPPORTED = -4,   /* shape is valid but no kernel is instantiated for it (never a silent no-op) */
     HW_ERR_FRAGMENTS = -5,     /* F < 1 or F > HW_MAX_FRAGMENTS */
     HW_ERR_WORKSPACE = -6,     /* workspace NULL or smaller than hw_workspace_bytes() */
@@ -116,6 +117,15 @@ int hw_workspace_bytes(const hw_problem* p, size_t* bytes);
 
 /* Rotate q per fragment in registers and attend; replaces hogwild_fused. */
 int hw_fused_attention(const hw_problem* p, void* stream);
+
+/* The two kernels of hw_fused_attention separately.  HW_STAGE_ATTENTION leaves the split-K partials of this
+   device's KV in the workspace (per kv head and workgroup: unnormalised output rows, running max in base-2 units
+   and sum); HW_STAGE_MERGE combines the partials found there into out / lse.  For a caller that holds only part of
+   the fragments and exchanges partials before merging, and for timing the attention kernel alone.  The reference
+   has the same split internally (kernel + reduce kernel, src/kernels/kernel_v21.cuh:985-989). */
+#define HW_STAGE_ATTENTION 1
+#define HW_STAGE_MERGE 2
+int hw_fused_attention_stages(const hw_problem* p, void* stream, int stages);
 
 /* Attend with already-rotated queries [F,W,Hq,S,E]; replaces hogwild_sdpa. */
 int hw_sdpa(const hw_problem* p, void* stream);

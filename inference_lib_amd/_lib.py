@@ -22,7 +22,7 @@ _DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_
 
 EXPORTS = [
     "hw_version", "hw_status_string", "hw_validate", "hw_plan_debug", "hw_workspace_bytes",
-    "hw_fused_attention", "hw_sdpa", "hw_rope", "hw_device_cus",
+    "hw_fused_attention", "hw_fused_attention_stages", "hw_sdpa", "hw_rope", "hw_device_cus",
     "hw_event_create", "hw_event_destroy", "hw_event_record", "hw_event_synchronize", "hw_event_elapsed_ms",
     "hw_stream_read", "hw_stream_copy",
 ]
@@ -73,6 +73,7 @@ def _load() -> C.CDLL:
     lib.hw_workspace_bytes.argtypes = [C.POINTER(HwProblem), C.POINTER(C.c_size_t)]
     lib.hw_fused_attention.argtypes = [C.POINTER(HwProblem), C.c_void_p]
     lib.hw_sdpa.argtypes = [C.POINTER(HwProblem), C.c_void_p]
+    lib.hw_fused_attention_stages.argtypes = [C.POINTER(HwProblem), C.c_void_p, C.c_int]
     lib.hw_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                             C.c_int, C.c_int, C.c_int, C.c_void_p]
     lib.hw_event_create.argtypes = [C.POINTER(C.c_void_p)]
@@ -207,11 +208,17 @@ class Problem:
         self.p.ev_start = start
         self.p.ev_stop = stop
 
-    def run(self) -> None:
+    def run(self, stages: int = 3) -> None:
+        """stages: 1 = attention kernel only (partials stay in the workspace), 2 = merge only, 3 = both."""
         if self._ws is None:
             self.set_workspace()
         with torch.cuda.device(self.device):
             stream = torch.cuda.current_stream(self.device).cuda_stream
+            if stages != 3:
+                if self.prerotated:
+                    raise ValueError("separate stages exist for the fused entry only")
+                check(lib.hw_fused_attention_stages(C.byref(self.p), C.c_void_p(stream), stages), "hw_fused_attention_stages")
+                return
             fn = lib.hw_sdpa if self.prerotated else lib.hw_fused_attention
             check(fn(C.byref(self.p), C.c_void_p(stream)), fn.__name__)
 

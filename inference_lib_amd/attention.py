@@ -54,10 +54,13 @@ def hogwild_sdpa(queries: torch.Tensor, locations: torch.Tensor, keys: List[torc
                           device=queries.device)
     keys = [k.contiguous() for k in keys]
     values = [v.contiguous() for v in values]
-    if HAVE_TORCH_OPS and lse is None:
+    if HAVE_TORCH_OPS:
         if fragment_lengths is None:
             fragment_lengths = torch.tensor([k.size(-2) for k in keys], dtype=torch.int32, device=queries.device)
-        torch.ops.libhogatt.hogwild_sdpa(out, scale, locations, queries.contiguous(), fragment_lengths, keys, values)
+        if lse is None:
+            torch.ops.libhogatt.hogwild_sdpa(out, scale, locations, queries.contiguous(), fragment_lengths, keys, values)
+        else:
+            torch.ops.libhogatt.hogwild_sdpa_lse(out, lse, scale, locations, queries.contiguous(), fragment_lengths, keys, values)
         return out
     pr = _lib.Problem(q=queries.contiguous(), locations=locations, keys=keys, values=values, scale=scale, out=out, lse=lse,
                       prerotated=True)

@@ -42,7 +42,7 @@ int validate(const hw_problem* p, int fused) {
     if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
     if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
     if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
-    if (!(p->scale == p->scale)) return HW_ERR_SHAPE;
+    if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return HW_ERR_SHAPE;   // the row max is taken before scaling
     if (fused) {
         if (p->RotE < 0 || p->RotE > p->E || (p->RotE & 1)) return HW_ERR_SHAPE;
     }
@@ -55,7 +55,8 @@ int validate(const hw_problem* p, int fused) {
         if (p->len[f] < 0) return HW_ERR_SHAPE;
         if (p->len[f] > 0 && (p->k[f] == nullptr || p->v[f] == nullptr)) return HW_ERR_NULL;
         if (!aligned16(p->k[f]) || !aligned16(p->v[f])) return HW_ERR_ALIGN;
-        if ((long long)p->len[f] * p->Hkv * p->E * (long long)elem_size(p->dtype) > (1ll << 40)) return HW_ERR_SHAPE;
+        // one kv head of a fragment is addressed through a 32-bit buffer offset
+        if ((long long)p->len[f] * (p->E > p->Ev ? p->E : p->Ev) * (long long)elem_size(p->dtype) >= 0x7fff0000ll) return HW_ERR_SHAPE;
     }
     if (!aligned16(p->out) || !aligned16(p->q)) return HW_ERR_ALIGN;
     if (fused && (!aligned16(p->cosines) || !aligned16(p->sines) || !aligned16(p->rq))) return HW_ERR_ALIGN;
@@ -154,7 +155,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
     return HW_OK;
 }
 
-int run(const hw_problem* p, void* stream_, int fused) {
+int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATTENTION | HW_STAGE_MERGE) {
     int st = validate(p, fused);
     if (st != HW_OK) return st;
     int cus = 0;
@@ -207,7 +208,8 @@ int run(const hw_problem* p, void* stream_, int fused) {
     ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
     ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
 
-    hipError_t e;
+    hipError_t e = hipSuccess;
+    if (stages & HW_STAGE_ATTENTION) {
     if (p->ev_start != nullptr) {
         e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_start), stream);
         if (e != hipSuccess) return (int)e;
@@ -218,6 +220,8 @@ int run(const hw_problem* p, void* stream_, int fused) {
         e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_stop), stream);
         if (e != hipSuccess) return (int)e;
     }
+    }
+    if (!(stages & HW_STAGE_MERGE)) return (int)e;
     hw::MergeArgs ma;
     ma.part_o = ka.h.part_o;
     ma.part_ml = ka.h.part_ml;
@@ -279,6 +283,11 @@ int hw_workspace_bytes(const hw_problem* p, size_t* bytes) {
 int hw_fused_attention(const hw_problem* p, void* stream) { return run(p, stream, 1); }
 
 int hw_sdpa(const hw_problem* p, void* stream) { return run(p, stream, 0); }
+
+int hw_fused_attention_stages(const hw_problem* p, void* stream, int stages) {
+    if ((stages & (HW_STAGE_ATTENTION | HW_STAGE_MERGE)) == 0 || (stages & ~(HW_STAGE_ATTENTION | HW_STAGE_MERGE)) != 0) return HW_ERR_SHAPE;
+    return run(p, stream, 1, stages);
+}
 
 int hw_rope(void* out, const void* q, const float* cosines, const float* sines, int dtype, int F, int W, int Hq, int S, int E,
             int RotE, void* stream) {

@@ -1,0 +1,158 @@
+"""Host-side checks of the C ABI that need no GPU: the shared library loads, exports every symbol the header
+declares, rejects bad arguments before touching a device, and plans the split sensibly."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _lib():
+    from inference_lib_amd import _lib
+    return _lib
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib()
+    header = open(os.path.join(ROOT, "include", "hogwild_hip.h")).read()
+    declared = set(re.findall(r"^\s*(?:int|const char\*)\s+(hw_\w+)\s*\(", header, flags=re.M))
+    assert declared, "no declarations found in the header"
+    assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
+    for name in declared:
+        assert hasattr(L.lib, name), name
+    assert L.lib.hw_version() == 1
+
+
+def test_struct_layout_matches_header():
+    """ctypes mirror and C struct must agree; sizeof is probed through a tiny C program when gcc is around."""
+    import shutil
+    import subprocess
+    import tempfile
+    L = _lib()
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "s.c")
+        open(src, "w").write('#include <stdio.h>\n#include <stddef.h>\n#include "hogwild_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu\\n",'
+                             'sizeof(hw_problem),sizeof(hw_plan),offsetof(hw_problem,workspace),offsetof(hw_problem,ev_start),'
+                             'offsetof(hw_plan,workspace_bytes));return 0;}\n')
+        exe = os.path.join(d, "s")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)
+        out = subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()
+    assert int(out[0]) == C.sizeof(L.HwProblem)
+    assert int(out[1]) == C.sizeof(L.HwPlan)
+    assert int(out[2]) == L.HwProblem.workspace.offset
+    assert int(out[3]) == L.HwProblem.ev_start.offset
+    assert int(out[4]) == L.HwPlan.workspace_bytes.offset
+
+
+def _problem(L, **over):
+    F = over.pop("F", 2)
+    p = L.HwProblem()
+    p.dtype, p.F, p.W, p.Hq, p.Hkv, p.S, p.E, p.Ev, p.RotE = L.HW_BF16, F, 2, 8, 2, 1, 128, 128, 128
+    p.scale = 0.1
+    fake = 0x1000                                   # never dereferenced on the host
+    for f in ("out", "q", "locations", "cosines", "sines"):
+        setattr(p, f, fake)
+    k = (C.c_void_p * F)(*[fake] * F)
+    lens = (C.c_int32 * F)(*([64] * F))
+    p.k = C.cast(k, C.POINTER(C.c_void_p))
+    p.v = C.cast(k, C.POINTER(C.c_void_p))
+    p.len = C.cast(lens, C.POINTER(C.c_int32))
+    p._keep = (k, lens)
+    for key, val in over.items():
+        setattr(p, key, val)
+    return p
+
+
+def test_validation_happens_on_the_host():
+    L = _lib()
+    v = lambda p, fused=1: L.lib.hw_validate(C.byref(p), fused)
+    assert v(_problem(L)) == 0
+    assert L.lib.hw_validate(None, 1) == -1
+    assert v(_problem(L, dtype=7)) == -2
+    assert v(_problem(L, Hq=7)) == -3                       # not a multiple of Hkv
+    assert v(_problem(L, W=0)) == -3
+    assert v(_problem(L, RotE=130)) == -3                   # wider than the head
+    assert v(_problem(L, RotE=63)) == -3                    # odd
+    assert v(_problem(L, scale=float("nan"))) == -3
+    assert v(_problem(L, scale=-1.0)) == -3
+    assert v(_problem(L, E=96, Ev=96, RotE=96)) == -4       # valid but not instantiated: a hard error, never silent
+    assert v(_problem(L, Ev=64)) == -4
+    assert v(_problem(L, F=33)) == -5
+    assert v(_problem(L, F=0)) == -5
+    assert v(_problem(L, out=None)) == -1
+    assert v(_problem(L, cosines=None)) == -1
+    assert v(_problem(L, cosines=None), fused=0) == 0       # the pre-rotated entry needs no tables
+    assert v(_problem(L, q=0x1004)) == -7                   # misaligned
+    p = _problem(L)
+    p.len[1] = -5
+    assert v(p) == -3
+    # the launching entry points run the same checks first, so these fail without any device present
+    assert L.lib.hw_fused_attention(C.byref(_problem(L, dtype=9)), None) == -2
+    assert L.lib.hw_sdpa(C.byref(_problem(L, Hq=7)), None) == -3
+    assert L.lib.hw_rope(None, None, None, None, L.HW_BF16, 1, 1, 1, 1, 128, 128, None) == -1
+    assert L.lib.hw_rope(0x1000, 0x1000, 0x1000, 0x1000, 5, 1, 1, 1, 1, 128, 128, None) == -2
+    assert b"fragment" in L.lib.hw_status_string(-5)
+    assert L.status_string(0) == "ok"
+
+
+@pytest.mark.parametrize("lens,kw", [
+    ([4096] + [2048] * 4 + [41, 16, 110, 73], dict(W=4, S=1, Hq=40, Hkv=8, Ev=128)),
+    ([2048, 1024, 1024], dict(W=2, S=1, Hq=28, Hkv=4, Ev=128)),
+    ([16384] + [3000, 17, 4000, 250, 1, 999, 2048, 3333] + [1] * 8, dict(W=8, S=1, Hq=32, Hkv=8, Ev=128)),
+    ([8192] + [2048] * 4, dict(W=4, S=4, Hq=64, Hkv=8, Ev=128)),
+    ([256, 64, 64], dict(W=2, S=1, Hq=8, Hkv=2, Ev=64)),
+    ([0, 5, 0], dict(W=1, S=1, Hq=2, Hkv=1, Ev=64)),
+    ([0], dict(W=1, S=1, Hq=2, Hkv=1, Ev=64)),
+    ([1] * 32, dict(W=2, S=1, Hq=4, Hkv=2, Ev=128)),
+])
+def test_plan_invariants(lens, kw):
+    L = _lib()
+    for cus in (1, 8, 256, 304):
+        for splits in (0, 1, 5, 1000):
+            pl = L.plan(lens, num_cus=cus, splits=splits, **kw)
+            G = kw["Hq"] // kw["Hkv"]
+            assert pl.rows == kw["W"] * kw["S"] * G
+            assert pl.row_blocks in (1, 2) and pl.row_groups * 16 * pl.row_blocks >= pl.rows
+            tiles = sum((x + 31) // 32 for x in lens)
+            assert pl.tiles_per_head == tiles
+            tb = list(pl.tile_begin)
+            assert tb[0] == 0 and tb[len(lens)] == tiles and all(a <= b for a, b in zip(tb, tb[1:]))
+            n = pl.wgs_per_head
+            assert 1 <= n <= 256 and n <= max(tiles, 1)
+            wb = list(pl.wg_tile_begin)[: n + 1]
+            assert wb[0] == 0 and wb[-1] == tiles
+            assert all(a < b for a, b in zip(wb, wb[1:])) or tiles == 0          # every workgroup owns at least one tile
+            assert pl.workgroups == n * kw["Hkv"] * pl.row_groups
+            assert pl.workspace_bytes >= kw["Hkv"] * n * pl.rows * (kw["Ev"] + 2) * 4
+
+
+def test_plan_spreads_tiny_fragments():
+    """Opening a fragment has a fixed cost, so a run of tiny fragments must not end up in one workgroup."""
+    L = _lib()
+    lens = [4096] + [2048] * 4 + [41, 16, 110, 73]
+    pl = L.plan(lens, W=4, S=1, Hq=40, Hkv=8, Ev=128, num_cus=256)
+    wb = list(pl.wg_tile_begin)[: pl.wgs_per_head + 1]
+    tb = list(pl.tile_begin)[: len(lens) + 1]
+    worst = 0
+    for a, b in zip(wb, wb[1:]):
+        worst = max(worst, sum(1 for f in range(len(lens)) if max(a, tb[f]) < min(b, tb[f + 1])))
+    assert worst <= 2
+
+
+def test_no_fallback_when_library_is_missing(tmp_path, monkeypatch):
+    """The product path must fail loudly without the HIP library: importing the ctypes layer from a copy of the
+    package that has no libhogwild_hip.so raises ImportError."""
+    import shutil
+    import subprocess
+    import sys
+    pkg = tmp_path / "inference_lib_amd"
+    pkg.mkdir()
+    for name in ("__init__.py", "_lib.py", "attention.py", "cases.py"):
+        shutil.copy(os.path.join(ROOT, "inference_lib_amd", name), pkg / name)
+    r = subprocess.run([sys.executable, "-c", "import inference_lib_amd.attention"], cwd=tmp_path, capture_output=True, text=True,
+                       env={**os.environ, "PYTHONPATH": str(tmp_path)})
+    assert r.returncode != 0 and "libhogwild_hip.so" in r.stderr
