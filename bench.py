@@ -29,9 +29,10 @@ if ROOT not in sys.path:
 PEAK_HBM_GBS = 8000.0   # MI355X published HBM3E bandwidth
 METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 workers"
 
-# HBM bytes per launch of the attention kernel on this workload measured with rocprofv3 --pmc
-# (FETCH_SIZE, WRITE_SIZE; scaled by a copy kernel of known size).  None until measured.
-MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": None}
+# HBM bytes per launch of the attention kernel measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in
+# separate runs, each scaled by what the same counter reads for the 256 MiB copy kernel this script launches:
+# 0.5 for FETCH_SIZE, 1.0 for WRITE_SIZE): 51.84 MB fetched + 3.03 MB written.  Workloads not measured: None.
+MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_870_000}
 
 
 def parse_args():
@@ -191,6 +192,12 @@ def main():
         e1.record(s_handle)
         torch.cuda.synchronize()
         stream_gbs = big.numel() * 5 / (e0.elapsed_ms(e1) * 1e-3) / 1e9
+        # a plain copy of known size (256 MiB read + 256 MiB written): the reference point that scales the
+        # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under rocprofv3 --pmc
+        half = 256 * 1024 * 1024
+        for _ in range(2):
+            _lib.check(_lib.lib.hw_stream_copy(big.data_ptr() + half, big.data_ptr(), half, C.c_void_p(s_handle)), "hw_stream_copy")
+        torch.cuda.synchronize()
         del big
 
     value = kv_bytes / (graph_us * 1e-6) / 1e9
