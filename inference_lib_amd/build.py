@@ -20,8 +20,10 @@ TORCH_EXT = os.path.join(HERE, "hogatt.abi3.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
-# packed fp32 VALU ops are switched off for every device compile of this library
-DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# packed fp32 VALU ops are switched off for every device compile of this library; MFMA accumulators are kept in
+# architectural VGPRs (the attention kernel touches them with VALU ops, and shuttling them to and from the
+# accumulation registers cost more instructions than the arithmetic)
+DEVICE_FLAGS = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
 def _run(cmd):

@@ -30,6 +30,13 @@ namespace hw {
 #ifndef HW_PF2
 #define HW_PF2 2
 #endif
+// waves per SIMD the two-row-block 16-bit kernels are register-budgeted for (tuning knob)
+#ifndef HW_MINW2
+#define HW_MINW2 1
+#endif
+#ifndef HW_VGPR_CAP
+#define HW_VGPR_CAP
+#endif
 
 // Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
 #ifdef HW_CLOCKS
@@ -218,8 +225,9 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
 template <int RB, int NOC>
 struct WaveState {
     f32x4 o[RB][NOC];
-    float m[RB];   // running max of scale*log2(e)*q.k
+    float m[RB];   // reference of the exponentials (base-2 units): within 2^8 below/above the running max
     float l[RB];   // lane-partial sum: this lane's quarter of the tokens
+    bool fresh;    // no tile accumulated yet (uniform over the wave)
 };
 
 // One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
@@ -270,32 +278,53 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const
             sacc[rb][tb] = acc;
         }
     }
-    float p[RB][8];
+    // Online softmax with a lazily updated reference: exponentials are taken against st.m, which only moves when
+    // a row's maximum exceeds it by more than 2^LAZY_LOG2 (then O and l of that row are rescaled).  Most tiles
+    // therefore leave the accumulators alone: no rescale multiplies, and O can stay in the MFMA accumulator
+    // registers.  p is at most 2^LAZY_LOG2, far inside the range of every storage type.
+    constexpr float LAZY_LOG2 = 8.0f;
+    float s[RB][8];
+    float mxs[RB];
+    bool need = false;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-        float s[8];
         float mx = NEG_BIG;
 #pragma unroll
         for (int idx = 0; idx < 8; ++idx) {
-            s[idx] = sacc[rb][idx >> 2][idx & 3];
-            if constexpr (MASKED) s[idx] = (t0 + slot_token(q, idx)) < lim[rb] ? s[idx] : NEG_BIG;
-            mx = fmaxf(mx, s[idx]);
+            s[rb][idx] = sacc[rb][idx >> 2][idx & 3];
+            if constexpr (MASKED) s[rb][idx] = (t0 + slot_token(q, idx)) < lim[rb] ? s[rb][idx] : NEG_BIG;
+            mx = fmaxf(mx, s[rb][idx]);
         }
-        mx = quarter_max(mx) * sc;                     // sc > 0: scaling commutes with the max
-        const float mnew = fmaxf(st.m[rb], mx);
-        const float alpha = fast_exp2(st.m[rb] - mnew);
-        st.m[rb] = mnew;
-        // a row that has seen nothing yet has mnew ~ -1e29; exponentiate against 0 so its masked slots give 0, not 1
-        const float mref = MASKED ? (mnew < -1.0e28f ? 0.f : mnew) : mnew;
+        mx = quarter_max(mx);
+        mxs[rb] = mx < -1.0e29f ? NEG_BIG : mx * sc;      // sc > 0: scaling commutes with the max; nothing visible stays NEG_BIG
+        need = need || (mxs[rb] > st.m[rb] + LAZY_LOG2);
+    }
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {        // uniform over the wave
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const float mnew = mxs[rb] > st.m[rb] + LAZY_LOG2 ? mxs[rb] : st.m[rb];
+            const float alpha = fast_exp2(st.m[rb] - mnew);   // 1 for rows that keep their reference
+            st.m[rb] = mnew;
+            st.l[rb] *= alpha;
+            if (!st.fresh) {                                  // before the first tile O is zero
+#pragma unroll
+                for (int c = 0; c < G::NOC; ++c) st.o[rb][c] *= alpha;
+            }
+        }
+    }
+    st.fresh = false;
+    float p[RB][8];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        // a row that has seen nothing yet keeps the reference NEG_BIG; exponentiate against 0 so its masked slots give 0
+        const float mref = MASKED ? (st.m[rb] < -1.0e29f ? 0.f : st.m[rb]) : st.m[rb];
         float psum = 0.f;
 #pragma unroll
         for (int idx = 0; idx < 8; ++idx) {
-            p[rb][idx] = fast_exp2(__builtin_fmaf(s[idx], sc, -mref));
+            p[rb][idx] = fast_exp2(__builtin_fmaf(s[rb][idx], sc, -mref));
             psum += p[rb][idx];
         }
-        st.l[rb] = st.l[rb] * alpha + psum;
-#pragma unroll
-        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] *= alpha;
+        st.l[rb] += psum;
     }
 
     if constexpr (G::SZ == 2) {
@@ -506,7 +535,7 @@ struct QueryRotation {
 // 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the tile registers too large.
 // PF = tiles a wave keeps in flight.  PRE = queries arrive rotated (hogwild_sdpa), else fused rotation.
 template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE>
-__global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelArgs args) {
+__global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     constexpr int ROWS = RB * 16;
     constexpr int SSTR = EV + 4;      // padded row stride of the epilogue exchange: rows land in different banks
@@ -594,6 +623,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 #pragma unroll
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
+    st.fresh = true;
 
     unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
 
@@ -744,14 +774,17 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 }
 
 // Merge the split-K partials of one (kv head, row): out = sum_g 2^(m_g - M) O_g / sum_g 2^(m_g - M) l_g.
+// Latency-bound, so everything a thread needs from global memory (its partial rows and their max/sum pairs) is
+// requested in one batch before the first use; each thread then folds its partials with a running reference of
+// its own, and the NPG partial groups are combined through LDS.
 template <class DT, int EV>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     typedef typename Elem<DT>::store_t store_t;
     constexpr int V4 = EV / 4;          // threads along the head dim (4 floats each)
     constexpr int NPG = 256 / V4;       // partial groups
+    constexpr int UN = 4;               // partials per thread and batch
     __shared__ __attribute__((aligned(16))) float red[NPG][EV];
-    __shared__ float wgt_lds[MAX_SPLITS];
-    __shared__ float red_m[4], red_l[4];
+    __shared__ float red_m[NPG], red_l[NPG];
 
     const int hkv = blockIdx.x / a.R;
     const int r = blockIdx.x - hkv * a.R;
@@ -760,70 +793,64 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     const int ns = a.wgs_per_head;
     const float* ml = a.part_ml + ((size_t)hkv * ns * a.R + r) * 2;
     const size_t mstride = (size_t)a.R * 2;
-
-    // one (max, sum) pair per thread, block-wide max and rescaled sum
-    float m_own[MAX_SPLITS / 256], l_own[MAX_SPLITS / 256];
-    float M = NEG_BIG;
-#pragma unroll
-    for (int k = 0; k < MAX_SPLITS / 256; ++k) {
-        const int s = tid + k * 256;
-        m_own[k] = NEG_BIG;
-        l_own[k] = 0.f;
-        if (s < ns) {
-            const f32x2 v = *reinterpret_cast<const f32x2*>(ml + s * mstride);
-            m_own[k] = v.x;
-            l_own[k] = v.y;
-        }
-        M = fmaxf(M, m_own[k]);
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
-    if ((tid & 63) == 0) red_m[tid >> 6] = M;
-    __syncthreads();
-    M = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
-    float Lsum = 0.f;
-#pragma unroll
-    for (int k = 0; k < MAX_SPLITS / 256; ++k) {
-        const int s = tid + k * 256;
-        const float wgt = fast_exp2(m_own[k] - M);
-        if (s < ns) wgt_lds[s] = wgt;
-        Lsum += l_own[k] * wgt;
-    }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) Lsum += __shfl_xor(Lsum, off, 64);
-    if ((tid & 63) == 0) red_l[tid >> 6] = Lsum;
-    __syncthreads();
-    Lsum = (red_l[0] + red_l[1]) + (red_l[2] + red_l[3]);
-
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     const float* po = a.part_o + ((size_t)hkv * ns * a.R + r) * EV + e4 * 4;
     const size_t ostride = (size_t)a.R * EV;
-    int s = pg;
-    for (; s + 3 * NPG < ns; s += 4 * NPG) {
-        const f32x4 o0 = *reinterpret_cast<const f32x4*>(po + (size_t)s * ostride);
-        const f32x4 o1 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + NPG) * ostride);
-        const f32x4 o2 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + 2 * NPG) * ostride);
-        const f32x4 o3 = *reinterpret_cast<const f32x4*>(po + (size_t)(s + 3 * NPG) * ostride);
-        acc += o0 * wgt_lds[s];
-        acc += o1 * wgt_lds[s + NPG];
-        acc += o2 * wgt_lds[s + 2 * NPG];
-        acc += o3 * wgt_lds[s + 3 * NPG];
+
+    float m_run = NEG_BIG, l_run = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = pg; s0 < ns; s0 += UN * NPG) {
+        f32x4 o[UN];
+        f32x2 mlv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int s = s0 + u * NPG;
+            const int sc = s < ns ? s : pg;                 // clamp: the loads stay unconditional
+            o[u] = *reinterpret_cast<const f32x4*>(po + (size_t)sc * ostride);
+            mlv[u] = *reinterpret_cast<const f32x2*>(ml + (size_t)sc * mstride);
+            if (s >= ns) mlv[u] = f32x2{NEG_BIG, 0.f};
+        }
+        float mb = m_run;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) mb = fmaxf(mb, mlv[u].x);
+        const float sc_old = fast_exp2(m_run - mb);
+        acc *= sc_old;
+        l_run *= sc_old;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const float w = fast_exp2(mlv[u].x - mb);
+            acc += o[u] * w;
+            l_run += mlv[u].y * w;
+        }
+        m_run = mb;
     }
-    for (; s < ns; s += NPG) acc += *reinterpret_cast<const f32x4*>(po + (size_t)s * ostride) * wgt_lds[s];
     *reinterpret_cast<f32x4*>(&red[pg][e4 * 4]) = acc;
+    if (e4 == 0) {
+        red_m[pg] = m_run;
+        red_l[pg] = l_run;
+    }
     __syncthreads();
     if (pg == 0) {
-        for (int k = 1; k < NPG; ++k) acc += *reinterpret_cast<const f32x4*>(&red[k][e4 * 4]);
-        const float inv = Lsum > 0.f ? 1.0f / Lsum : 0.f;
+        float M = red_m[0];
+#pragma unroll
+        for (int k = 1; k < NPG; ++k) M = fmaxf(M, red_m[k]);
+        f32x4 tot = {0.f, 0.f, 0.f, 0.f};
+        float L = 0.f;
+#pragma unroll
+        for (int k = 0; k < NPG; ++k) {
+            const float w = fast_exp2(red_m[k] - M);
+            tot += *reinterpret_cast<const f32x4*>(&red[k][e4 * 4]) * w;
+            L += red_l[k] * w;
+        }
+        const float inv = L > 0.f ? 1.0f / L : 0.f;
         const int GQ = a.Hq / a.Hkv;
         const int ws = r / GQ, gq = r - ws * GQ;
         const int w = ws / a.S, sq = ws - w * a.S;
         const size_t orow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + sq);
         store_t* op = reinterpret_cast<store_t*>(a.out) + orow * EV + e4 * 4;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) op[i] = Elem<DT>::from_float(acc[i] * inv);
+        for (int i = 0; i < 4; ++i) op[i] = Elem<DT>::from_float(tot[i] * inv);
         if (a.lse != nullptr && e4 == 0)
-            a.lse[orow] = Lsum > 0.f ? (M + __builtin_amdgcn_logf(Lsum)) * 0.69314718055994530942f : -__builtin_inff();
+            a.lse[orow] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * 0.69314718055994530942f : -__builtin_inff();
     }
 }
 
@@ -881,7 +908,7 @@ static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t 
         hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
                            stream, ka);
     else
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1, half ? HW_PF2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, half ? HW_MINW2 : 1, half ? HW_PF2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
     return hipGetLastError();
 }
 
