@@ -50,7 +50,8 @@ int validate(const hw_problem* p, int fused) {
     if (p->k == nullptr || p->v == nullptr || p->len == nullptr) return HW_ERR_NULL;
     if (fused && p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
     long long rows = (long long)p->W * p->S * (p->Hq / p->Hkv);
-    if (rows > (1 << 20)) return HW_ERR_SHAPE;
+    if (rows >= (1 << 20) || p->S >= (1 << 12) || p->Hq / p->Hkv >= (1 << 12)) return HW_ERR_SHAPE;
+    if ((long long)p->Hkv * ((rows + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
     for (int f = 0; f < p->F; ++f) {
         if (p->len[f] < 0) return HW_ERR_SHAPE;
         if (p->len[f] > 0 && (p->k[f] == nullptr || p->v[f] == nullptr)) return HW_ERR_NULL;
@@ -207,6 +208,12 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     ka.h.prerotated = prerotated ? 1 : 0;
     ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
     ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
+    // multipliers for the in-kernel divisions (exact for numerators < 2^20 and divisors < 2^12, both validated)
+    auto magic = [](int d) { return (unsigned)(((1ull << 32) + (unsigned long long)d - 1) / (unsigned long long)d); };
+    ka.h.magic_gq = magic(p->Hq / p->Hkv);
+    ka.h.magic_s = magic(p->S);
+    ka.h.magic_nrg = magic(plan.row_groups);
+    ka.h.magic_wg = magic(plan.wgs_per_head);
 
     hipError_t e = hipSuccess;
     if (stages & HW_STAGE_ATTENTION) {

@@ -36,7 +36,7 @@ struct alignas(64) KernelHeader {
     int prerotated;
     int xcd_remap;
     float sc;           // scale * log2(e)
-    int pad[4];
+    unsigned magic_gq, magic_s, magic_nrg, magic_wg;   // ceil(2^32 / d) for d = Hq/Hkv, S, nrg, wgs_per_head
 };
 static_assert(sizeof(KernelHeader) == 128, "KernelHeader must be 32 dwords");
 

@@ -433,9 +433,13 @@ struct DevHeader {
     int prerotated;
     int xcd_remap;
     float sc;
-    int pad[4];
+    unsigned magic_gq, magic_s, magic_nrg, magic_wg;
 };
 static_assert(sizeof(DevHeader) == sizeof(KernelHeader), "DevHeader mirrors KernelHeader");
+
+// n / d for n < 2^20, d < 2^12 with the host-computed multiplier ceil(2^32 / d) mod 2^32: one multiply-high instead
+// of the ~25-instruction integer division sequence.  d == 1 gives the multiplier 0, which stands for "n itself".
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 
 // row r (0..R) of a kv head -> (worker*S + token, q head, flat q row index)
 struct RowMap {
@@ -444,9 +448,9 @@ struct RowMap {
 };
 __device__ __forceinline__ RowMap map_row(const DevHeader& a, int r, int hkv, int GQ) {
     RowMap m;
-    m.ws = r / GQ;
+    m.ws = fast_div(r, a.magic_gq);
     const int gq = r - m.ws * GQ;
-    const int w = m.ws / a.S, s = m.ws - w * a.S;
+    const int w = fast_div(m.ws, a.magic_s), s = m.ws - w * a.S;
     m.qrow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
     return m;
 }
@@ -565,13 +569,11 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     const int n = lane & 15;
     const int q = lane >> 4;
     char* const kslots[3] = {slot0.k + wv * G::KSTAGE, slot1 + (PF > 1 ? wv * G::KSTAGE : 0), slot2 + (PF > 2 ? wv * G::KSTAGE : 0)};
-    unsigned koff[G::KL];
-    k_lane_offsets<G>(koff, lane);
-
     // Everything the kernel needs from its arguments is requested here in one burst, before anything waits:
     // the fragment table and the workgroup boundary table with one vector load per lane and array, the 32
     // scalar dwords with two 64-byte scalar loads.  The argument segment is slow to reach and the compiler
-    // would otherwise fetch it lazily, one dependent round trip after another.
+    // would otherwise fetch it lazily, one dependent round trip after another.  The setup that does not depend
+    // on the arguments runs while they are in flight.
     const int fl = lane & (MAXF - 1);
     const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
     const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
@@ -589,19 +591,29 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     HeaderBits hb;
     {
         const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
-        asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40\n\ts_waitcnt lgkmcnt(0)"
-                     : "=&s"(hb.lo), "=&s"(hb.hi)
-                     : "s"(argp)
-                     : "memory");
+        asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(hb.lo), "=&s"(hb.hi) : "s"(argp) : "memory");
     }
+    unsigned koff[G::KL];
+    k_lane_offsets<G>(koff, lane);
+    WaveState<RB, G::NOC> st;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        st.m[rb] = NEG_BIG;
+        st.l[rb] = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    st.fresh = true;
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");   // the header is usable from here on
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
 
     // consecutive logical ids stay on one XCD (hardware deals workgroups round-robin over the 8 XCDs)
     int bid = blockIdx.x;
     if (a.xcd_remap) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
-    const int rg = bid % a.nrg;
-    const int g = (bid / a.nrg) % a.wgs_per_head;
-    const int hkv = bid / (a.nrg * a.wgs_per_head);
+    const int hg = fast_div(bid, a.magic_nrg);            // (kv head, split) pair
+    const int rg = bid - hg * a.nrg;
+    const int hkv = fast_div(hg, a.magic_wg);
+    const int g = hg - hkv * a.wgs_per_head;
 
     int T0 = 0, T1 = 0;
 #pragma unroll
@@ -615,16 +627,6 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     const int GQ = a.Hq / a.Hkv;
 
     HW_MARK(0);
-    WaveState<RB, G::NOC> st;
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        st.m[rb] = NEG_BIG;
-        st.l[rb] = 0.f;
-#pragma unroll
-        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    st.fresh = true;
-
     unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
 
     while (todo != 0) {
@@ -647,7 +649,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
         QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
         qrot.load(a, f, hkv, r0, GQ, tid);
         // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
-        const int lm = a.loc[(size_t)f * a.W * a.S + min(r0 + (tid & (ROWS - 1)), a.R - 1) / GQ];
+        const int lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
         // the first tile is requested before the prologue, further look-ahead tiles after it: a wave stalls
         // while the memory pipeline accepts its requests, and the prologue should not sit behind that stall
         TileRegs<DT, E, EV> tr[PF];
