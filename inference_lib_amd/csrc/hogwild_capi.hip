@@ -236,6 +236,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     ma.lse = p->lse;
     ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = plan.rows;
     ma.wgs_per_head = plan.wgs_per_head;
+    ma.xcd_local = (plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
     e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
     return (int)e;
 }

@@ -52,6 +52,7 @@ struct MergeArgs {
     void* out;
     float* lse;
     int W, Hq, Hkv, S, R, wgs_per_head;
+    int xcd_local;      // kv head h was computed on XCD h / (Hkv/8): merge it there
 };
 
 hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream);

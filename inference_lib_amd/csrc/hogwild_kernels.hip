@@ -646,8 +646,10 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
 
         // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first PF
         // K/V tiles; the rotation then waits only for the former while the tiles stay in flight
+        HW_MARK(6);
         QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
         qrot.load(a, f, hkv, r0, GQ, tid);
+        HW_MARK(7);
         // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
         const int lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
         // the first tile is requested before the prologue, further look-ahead tiles after it: a wave stalls
@@ -788,8 +790,18 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     __shared__ __attribute__((aligned(16))) float red[NPG][EV];
     __shared__ float red_m[NPG], red_l[NPG];
 
-    const int hkv = blockIdx.x / a.R;
-    const int r = blockIdx.x - hkv * a.R;
+    // Workgroups are dealt round-robin over the 8 XCDs.  When the attention kernel kept each kv head on one XCD, merge
+    // that head's rows on the same XCD: its partials are then still in that XCD's L2.
+    int hkv, r;
+    if (a.xcd_local) {
+        const int hpx = a.Hkv >> 3;                       // heads per XCD
+        const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
+        hkv = x * hpx + j % hpx;
+        r = j / hpx;
+    } else {
+        hkv = blockIdx.x / a.R;
+        r = blockIdx.x - hkv * a.R;
+    }
     const int tid = threadIdx.x;
     const int e4 = tid % V4, pg = tid / V4;
     const int ns = a.wgs_per_head;
