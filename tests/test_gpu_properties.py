@@ -1,0 +1,201 @@
+"""Properties of the HIP path that hold at any size, checked on the GPU through the C ABI: independence of the
+split plan, of fragment order and of fragment splitting, determinism, empty rows / empty fragments, the fragment
+limit, streams and HIP-graph replay, and the two stages run separately."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np64, oracle_fused, run_fused
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available()
+    return torch.device("cuda:0")
+
+
+def _problem(cd, out, *, rq=None, lse=None, **kw):
+    from inference_lib_amd import _lib
+    return _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out,
+                        cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse, **kw)
+
+
+def test_split_plan_does_not_change_the_result(oracle):
+    """Any number of workgroups per head and either row-block setting gives the same answer up to fp32
+    accumulation order, at the full size of the headline workload."""
+    from inference_lib_amd import cases
+    c = cases.baseline_case(3)
+    cd = c.to(_dev())
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    W, Hq, S, E = cd.q.shape
+    base = None
+    for splits, rb in [(0, 0), (1, 0), (3, 0), (17, 0), (64, 0), (256, 0), (0, 1), (5, 1)]:
+        print(f"splits={splits} row_blocks={rb}", flush=True)
+        out = torch.empty((W, Hq, S, E), dtype=cd.q.dtype, device=_dev())
+        lse = torch.empty((W, Hq, S), dtype=torch.float32, device=_dev())
+        _problem(cd, out, lse=lse, splits=splits, row_blocks=rb).run()
+        torch.cuda.synchronize()
+        assert_close("out", out, o_ref, TOL[c.dtype])
+        assert_close("lse", lse, l_ref, TOL[c.dtype])
+        if base is None:
+            base = (out.clone(), lse.clone())
+        else:
+            assert (out.float() - base[0].float()).abs().max().item() <= 2 ** -7      # one bf16 ulp at |x| < 1 is 2^-8
+            assert (lse - base[1]).abs().max().item() <= 1e-4
+
+
+def test_runs_are_bit_identical():
+    from inference_lib_amd import cases
+    cd = cases.baseline_case(2).to(_dev())
+    a = run_fused(cd)
+    b = run_fused(cd)
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+
+
+def test_fragment_order_and_fragment_split_invariance(oracle):
+    from inference_lib_amd import cases
+    c = cases.small_case(dtype="f32", W=2, S=2, Hq=4, Hkv=2, E=64, lens=(150, 70, 90), seed=13)
+    cd = c.to(_dev())
+    out, lse, _ = run_fused(cd)
+    # reorder the fragments
+    perm = [2, 0, 1]
+    c2 = cases.small_case(dtype="f32", W=2, S=2, Hq=4, Hkv=2, E=64, lens=(150, 70, 90), seed=13)
+    c2.keys = [c.keys[i] for i in perm]
+    c2.values = [c.values[i] for i in perm]
+    c2.lens = [c.lens[i] for i in perm]
+    c2.locations = c.locations[perm].contiguous()
+    c2.cos = c.cos[perm].contiguous()
+    c2.sin = c.sin[perm].contiguous()
+    out2, lse2, _ = run_fused(c2.to(_dev()))
+    assert (out - out2).abs().max().item() < 1e-5 and (lse - lse2).abs().max().item() < 1e-5
+    # cut fragment 0 at token 37 with pre-rotated queries (only the mask bound moves: loc2 = loc - 37)
+    from inference_lib_amd import _lib
+    rq = torch.empty((c.F, 2, 4, 2, 64), dtype=torch.float32, device=_dev())
+    _lib.rope(cd.q, cd.cos, cd.sin, rq)
+    L1 = 37
+    keys = [cd.keys[0][:, :L1].contiguous(), cd.keys[0][:, L1:].contiguous()] + cd.keys[1:]
+    vals = [cd.values[0][:, :L1].contiguous(), cd.values[0][:, L1:].contiguous()] + cd.values[1:]
+    loc = torch.cat([cd.locations[:1], cd.locations[:1] - L1, cd.locations[1:]]).contiguous()
+    rq2 = torch.cat([rq[:1], rq[:1], rq[1:]]).contiguous()
+    out3 = torch.empty_like(out)
+    lse3 = torch.empty_like(lse)
+    _lib.Problem(q=rq2, locations=loc, keys=keys, values=vals, scale=c.scale, out=out3, lse=lse3, prerotated=True).run()
+    torch.cuda.synchronize()
+    assert (out - out3).abs().max().item() < 1e-5 and (lse - lse3).abs().max().item() < 1e-5
+
+
+def test_rows_that_see_nothing_and_empty_fragments(oracle):
+    """A worker whose locations are all -1 gets zeros and lse = -inf (the kernel's convention,
+    kernel_v21.cuh:238-245,627-629); zero-length fragments are legal and their rotated queries are still written."""
+    from inference_lib_amd import cases
+    c = cases.small_case(dtype="bf16", W=3, S=1, Hq=6, Hkv=2, E=128, lens=(70, 0, 33, 40), seed=17)
+    c.locations[:, 2, :] = -1                      # worker 2 sees nothing at all
+    cd = c.to(_dev())
+    out, lse, rq = run_fused(cd)
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL["bf16"])
+    assert_close("lse", lse, l_ref, TOL["bf16"])
+    assert torch.all(out[2] == 0) and torch.all(torch.isneginf(lse[2]))
+    assert_close("rq incl. the empty fragment", rq, rq_ref, 3.2e-2)
+
+
+def test_fragment_limit(oracle):
+    from inference_lib_amd import _lib, cases
+    lens = [40] + [3 + (i % 5) for i in range(31)]
+    W = 31
+    c = cases.build_case("f32max", "bf16", W, 1, 2 * W // W * 2, 2, 64, 1e4, lens, [[0, 1 + w] for w in range(W)],
+                         torch.Generator().manual_seed(3))
+    assert c.F == 32
+    out, lse, _ = run_fused(c.to(_dev()))
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL["bf16"])
+    assert_close("lse", lse, l_ref, TOL["bf16"])
+    with pytest.raises(_lib.HogwildError) as ei:
+        cd = c.to(_dev())
+        loc = torch.cat([cd.locations, cd.locations[:1]]).contiguous()
+        cs = torch.cat([cd.cos, cd.cos[:1]]).contiguous()
+        _lib.Problem(q=cd.q, locations=loc, keys=cd.keys + cd.keys[:1], values=cd.values + cd.values[:1], scale=c.scale,
+                     out=torch.empty_like(out), cosines=cs, sines=cs)
+    assert ei.value.status == -5
+
+
+def test_long_fragment_many_tiles_per_workgroup(oracle):
+    """One kv head and a 150k-token fragment: every workgroup walks hundreds of tiles; S=3 gives a causal tail."""
+    from inference_lib_amd import cases
+    g = torch.Generator().manual_seed(5)
+    c = cases.build_case("long", "f16", 1, 3, 4, 1, 128, 1e6, [150_001, 77], [[0, 1]], g)
+    out, lse, _ = run_fused(c.to(_dev()))
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL["f16"])
+    assert_close("lse", lse, l_ref, TOL["f16"])
+
+
+def test_two_stages_equal_the_fused_call():
+    from inference_lib_amd import cases
+    cd = cases.baseline_case(2).to(_dev())
+    W, Hq, S, E = cd.q.shape
+    out1 = torch.empty((W, Hq, S, E), dtype=cd.q.dtype, device=_dev())
+    out2 = torch.full_like(out1, float("nan"))
+    lse1 = torch.empty((W, Hq, S), dtype=torch.float32, device=_dev())
+    lse2 = torch.full_like(lse1, float("nan"))
+    _problem(cd, out1, lse=lse1).run()
+    pr = _problem(cd, out2, lse=lse2)
+    pr.run(stages=1)
+    torch.cuda.synchronize()
+    assert torch.isnan(out2.float()).all()          # the attention stage alone does not touch the output
+    pr.run(stages=2)
+    torch.cuda.synchronize()
+    assert torch.equal(out1, out2) and torch.equal(lse1, lse2)
+
+
+def test_side_stream_and_concurrent_streams(oracle):
+    from inference_lib_amd import cases
+    ca = cases.small_case(dtype="bf16", W=2, S=1, Hq=8, Hkv=2, E=128, lens=(900, 300, 411), seed=31)
+    cb = cases.small_case(dtype="f16", W=2, S=2, Hq=4, Hkv=2, E=64, lens=(500, 123, 77), seed=32)
+    da, db = ca.to(_dev()), cb.to(_dev())
+    oa = torch.empty((2, 8, 1, 128), dtype=torch.bfloat16, device=_dev())
+    ob = torch.empty((2, 4, 2, 64), dtype=torch.float16, device=_dev())
+    pa, pb = _problem(da, oa), _problem(db, ob)
+    pa.set_workspace()
+    pb.set_workspace()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for _ in range(5):
+        with torch.cuda.stream(sa):
+            pa.run()
+        with torch.cuda.stream(sb):
+            pb.run()
+    torch.cuda.synchronize()
+    assert_close("stream a", oa, oracle_fused(oracle, ca)[0], TOL["bf16"])
+    assert_close("stream b", ob, oracle_fused(oracle, cb)[0], TOL["f16"])
+
+
+def test_graph_replay_matches_eager():
+    """Captured once, replayed several times with eager launches and synchronisations in between; the inputs
+    change between replays and every replay must equal the eager result on the same inputs."""
+    from inference_lib_amd import cases
+    cd = cases.baseline_case(2).to(_dev())
+    W, Hq, S, E = cd.q.shape
+    out_g = torch.empty((W, Hq, S, E), dtype=cd.q.dtype, device=_dev())
+    out_e = torch.empty_like(out_g)
+    pg, pe = _problem(cd, out_g), _problem(cd, out_e)
+    pg.set_workspace()
+    pe.set_workspace()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        pg.run()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            pg.run()
+    for it in range(4):
+        cd.q.mul_(1.0 + 0.25 * it)                  # same buffers, new contents
+        cd.keys[1].add_(0.125)
+        torch.cuda.synchronize()
+        out_g.fill_(float("nan"))
+        graph.replay()
+        pe.run()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e), f"replay {it} differs from the eager launch"
