@@ -15,6 +15,13 @@
  *   hw_problem ............. struct Shape + the launcher argument list, src/common.h:5-20,
  *                            src/kernels/kernel_v21.cuh:951-957
  *   hw_status / hw_status_string ... cudaError_t + CUDA_RETURN_ON_ERROR, src/cuda_check.cuh:6-29
+ *   hw_paged_sdpa .......... hogwild_paged_sdpa       src/binding.cu:110-142, :269-281 (schema :369-370)
+ *                            + launcher v21::hogwild_paged_attention_gpu, src/kernels/kernel_v21.cuh:998-1043
+ *   hw_varlen_paged_sdpa ... hogwild_varlen_paged_sdpa  src/binding.cu:144-181, :283-296 (schema :373-374)
+ *                            + launcher v21::hogwild_varlen_paged_attention_gpu, src/kernels/kernel_v21.cuh:1045-1086
+ *   hw_copy_to_blocks ...... copy_to_blocks           src/binding.cu:183-215, :310-322 (schema :371-372);
+ *                            kernel src/cache.cuh:6-49
+ *   hw_paged_problem ....... struct Shape with its paged / varlen members, src/common.h:5-20
  */
 #ifndef HOGWILD_HIP_H
 #define HOGWILD_HIP_H
@@ -133,6 +140,93 @@ int hw_sdpa(const hw_problem* p, void* stream);
 /* out[F,W,Hq,S,E] = rope(q[W,Hq,S,E], cos/sin[F,W,S,RotE]); replaces hogwild_rope. */
 int hw_rope(void* out, const void* q, const float* cosines, const float* sines, int dtype,
             int F, int W, int Hq, int S, int E, int RotE, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Paged variants: the KV of worker (sequence) w lives in blocks of one cache tensor and is found through a block
+ * table (src/kernels/kernel_v21.cuh:405-411).  Every fragment f attends the same sequence from position 0 with its
+ * own queries and its own bound min(fragment_lengths, location + 1) (kernel_v21.cuh:385-388).
+ *
+ *   key_cache   [num_blocks, Hkv, block_size, E]    dtype
+ *   value_cache [num_blocks, Hkv, block_size, Ev]   dtype
+ *   block_table [W, max_blocks]                     int32; position l of sequence w is row l % block_size of block
+ *                                                   block_table[w][l / block_size].  Entries are clamped into
+ *                                                   0..num_blocks-1 on the device (a corrupt table reads wrong rows
+ *                                                   but never outside the cache).
+ * fixed-length operator (cu_seqlens_q == NULL), hw_paged_sdpa:
+ *   q [F, W, Hq, S, E] rotated, locations [F, W, S], fragment_lengths [F] (device), out [W, Hq, S, Ev], lse [W, Hq, S]
+ * packed variable-length operator (cu_seqlens_q != NULL), hw_varlen_paged_sdpa:
+ *   q [F, total_q, Hq, E] rotated, locations [F, total_q], fragment_lengths [F, W] (device), cu_seqlens_q [W + 1]
+ *   (device; query tokens cu[w] .. cu[w+1]-1 belong to sequence w, kernel_v21.cuh:15-23), out [total_q, Hq, Ev],
+ *   lse [total_q, Hq].  S is ignored.
+ * Nothing is read from a sequence beyond what some query row can see, so the lengths need not be known on the host.
+ * Limits: block_size < 4096, block_size * max_blocks <= 2^20 positions per sequence, num_blocks * Hkv * block_size
+ * < 2^31 cache rows, query rows per kv head (tokens * Hq/Hkv) < 2^20.
+ */
+typedef struct hw_paged_problem {
+    int32_t dtype;
+    int32_t F, W, Hq, Hkv, E, Ev;
+    int32_t S;                 /* query tokens per worker (fixed-length operator) */
+    int32_t total_q;           /* packed query tokens over all workers (variable-length operator) */
+    int32_t block_size, max_blocks, num_blocks;
+    float scale;
+    void* out;
+    float* lse;                /* optional */
+    const void* q;
+    const int32_t* locations;
+    const int32_t* fragment_lengths;
+    const void* key_cache;
+    const void* value_cache;
+    const int32_t* block_table;
+    const int32_t* cu_seqlens_q;   /* NULL selects the fixed-length operator */
+    void* workspace;
+    size_t workspace_bytes;
+    int32_t splits;            /* 0 = automatic; otherwise workgroups per (kv head, row group) */
+    int32_t row_blocks;        /* 0 = automatic; 1 or 2 = 16-row MFMA blocks per workgroup */
+} hw_paged_problem;
+
+typedef struct hw_paged_plan {
+    int32_t rows;              /* query rows per kv head: tokens * Hq/Hkv */
+    int32_t row_blocks;
+    int32_t row_groups;        /* over all workers; an upper bound for the variable-length operator */
+    int32_t splits;            /* workgroups per (kv head, row group); tile t of a sequence goes to wave t mod (4 * splits) */
+    int32_t workgroups;
+    size_t workspace_bytes;
+} hw_paged_plan;
+
+int hw_paged_validate(const hw_paged_problem* p);
+int hw_paged_plan_debug(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan);   /* host only */
+int hw_paged_workspace_bytes(const hw_paged_problem* p, size_t* bytes);
+/* replaces hogwild_paged_sdpa (cu_seqlens_q must be NULL) */
+int hw_paged_sdpa(const hw_paged_problem* p, void* stream);
+/* replaces hogwild_varlen_paged_sdpa (cu_seqlens_q must not be NULL) */
+int hw_varlen_paged_sdpa(const hw_paged_problem* p, void* stream);
+/* either operator, attention kernel and merge kernel separately (HW_STAGE_*), for timing */
+int hw_paged_sdpa_stages(const hw_paged_problem* p, void* stream, int stages);
+
+/*
+ * Append new K/V rows to the paged caches: token t of sequence b goes to position seq_lengths[b] + t of that
+ * sequence (src/cache.cuh:29-48).  key_states / value_states are [B, Hkv, S_new, E|Ev] with element strides
+ * (ks_*, vs_*) for the first three dimensions and a contiguous last dimension, so the usual transposed view of a
+ * [B, S_new, Hkv, D] projection can be passed as it is.  block_table [B, max_blocks], seq_lengths [B]: device int32.
+ * A position outside the block table, or a table entry outside the cache, is skipped (the reference would write out
+ * of bounds).  The reference launches S_new * max(E, Ev) threads per block and therefore cannot take more than
+ * 8 new tokens at head dimension 128 (src/binding.cu:201-203); there is no such limit here.
+ */
+typedef struct hw_copy_blocks {
+    int32_t dtype;
+    int32_t B, Hkv, S_new, E, Ev;
+    int32_t block_size, max_blocks, num_blocks;
+    const void* key_states;
+    const void* value_states;
+    int64_t ks_b, ks_h, ks_s;
+    int64_t vs_b, vs_h, vs_s;
+    void* key_cache;
+    void* value_cache;
+    const int32_t* block_table;
+    const int32_t* seq_lengths;
+} hw_copy_blocks;
+
+int hw_copy_to_blocks(const hw_copy_blocks* c, void* stream);
 
 /* Number of compute units of the current device (0 on failure). */
 int hw_device_cus(void);

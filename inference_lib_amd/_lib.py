@@ -25,6 +25,8 @@ EXPORTS = [
     "hw_fused_attention", "hw_fused_attention_stages", "hw_sdpa", "hw_rope", "hw_device_cus",
     "hw_event_create", "hw_event_destroy", "hw_event_record", "hw_event_synchronize", "hw_event_elapsed_ms",
     "hw_stream_read", "hw_stream_copy",
+    "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
+    "hw_paged_sdpa_stages", "hw_copy_to_blocks",
 ]
 
 
@@ -50,6 +52,41 @@ class HwPlan(C.Structure):
         ("tile_begin", C.c_int32 * (HW_MAX_FRAGMENTS + 1)),
         ("wg_tile_begin", C.c_int32 * (HW_MAX_SPLITS + 1)),
         ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class HwPagedProblem(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("F", C.c_int32), ("W", C.c_int32), ("Hq", C.c_int32), ("Hkv", C.c_int32), ("E", C.c_int32), ("Ev", C.c_int32),
+        ("S", C.c_int32), ("total_q", C.c_int32),
+        ("block_size", C.c_int32), ("max_blocks", C.c_int32), ("num_blocks", C.c_int32),
+        ("scale", C.c_float),
+        ("out", C.c_void_p), ("lse", C.c_void_p), ("q", C.c_void_p), ("locations", C.c_void_p),
+        ("fragment_lengths", C.c_void_p), ("key_cache", C.c_void_p), ("value_cache", C.c_void_p),
+        ("block_table", C.c_void_p), ("cu_seqlens_q", C.c_void_p),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("splits", C.c_int32), ("row_blocks", C.c_int32),
+    ]
+
+
+class HwPagedPlan(C.Structure):
+    _fields_ = [
+        ("rows", C.c_int32), ("row_blocks", C.c_int32), ("row_groups", C.c_int32), ("splits", C.c_int32),
+        ("workgroups", C.c_int32), ("workspace_bytes", C.c_size_t),
+    ]
+
+
+class HwCopyBlocks(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32),
+        ("B", C.c_int32), ("Hkv", C.c_int32), ("S_new", C.c_int32), ("E", C.c_int32), ("Ev", C.c_int32),
+        ("block_size", C.c_int32), ("max_blocks", C.c_int32), ("num_blocks", C.c_int32),
+        ("key_states", C.c_void_p), ("value_states", C.c_void_p),
+        ("ks_b", C.c_int64), ("ks_h", C.c_int64), ("ks_s", C.c_int64),
+        ("vs_b", C.c_int64), ("vs_h", C.c_int64), ("vs_s", C.c_int64),
+        ("key_cache", C.c_void_p), ("value_cache", C.c_void_p),
+        ("block_table", C.c_void_p), ("seq_lengths", C.c_void_p),
     ]
 
 
@@ -83,6 +120,13 @@ def _load() -> C.CDLL:
     lib.hw_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     lib.hw_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     lib.hw_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.hw_paged_validate.argtypes = [C.POINTER(HwPagedProblem)]
+    lib.hw_paged_plan_debug.argtypes = [C.POINTER(HwPagedProblem), C.c_int, C.POINTER(HwPagedPlan)]
+    lib.hw_paged_workspace_bytes.argtypes = [C.POINTER(HwPagedProblem), C.POINTER(C.c_size_t)]
+    lib.hw_paged_sdpa.argtypes = [C.POINTER(HwPagedProblem), C.c_void_p]
+    lib.hw_varlen_paged_sdpa.argtypes = [C.POINTER(HwPagedProblem), C.c_void_p]
+    lib.hw_paged_sdpa_stages.argtypes = [C.POINTER(HwPagedProblem), C.c_void_p, C.c_int]
+    lib.hw_copy_to_blocks.argtypes = [C.POINTER(HwCopyBlocks), C.c_void_p]
     return lib
 
 
@@ -237,6 +281,172 @@ def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num
     out = HwPlan()
     check(lib.hw_plan_debug(C.byref(p), num_cus, C.byref(out)), "hw_plan_debug")
     return out
+
+
+class PagedProblem:
+    """One call of the paged attention operators (hw_paged_sdpa, or hw_varlen_paged_sdpa when cu_seqlens_q is given).
+
+    fixed length:    q [F, W, Hq, S, E], locations [F, W, S], fragment_lengths [F], out [W, Hq, S, Ev], lse [W, Hq, S]
+    variable length: q [F, T, Hq, E], locations [F, T], fragment_lengths [F, W], cu_seqlens_q [W+1], out [T, Hq, Ev],
+                     lse [T, Hq]
+    key_cache / value_cache [num_blocks, Hkv, block_size, E|Ev], block_table int32 [W, max_blocks].
+    """
+
+    def __init__(self, *, q: torch.Tensor, locations: torch.Tensor, fragment_lengths: torch.Tensor,
+                 key_cache: torch.Tensor, value_cache: torch.Tensor, block_table: torch.Tensor, scale: float,
+                 out: torch.Tensor, cu_seqlens_q: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                 splits: int = 0, row_blocks: int = 0):
+        varlen = cu_seqlens_q is not None
+        if out.dtype not in _DTYPE_CODE:
+            raise HogwildError(-2, "PagedProblem")
+        if key_cache.dim() != 4 or value_cache.dim() != 4 or key_cache.shape[:3] != value_cache.shape[:3]:
+            raise ValueError("key_cache / value_cache must be [num_blocks, Hkv, block_size, E|Ev]")
+        NB, Hkv, BS, E = key_cache.shape
+        Ev = value_cache.size(3)
+        if block_table.dim() != 2:
+            raise ValueError("block_table must be [W, max_blocks]")
+        W = block_table.size(0)
+        F = locations.size(0)
+        if varlen:
+            T, Hq = out.size(0), out.size(1)
+            S = 0
+            if tuple(out.shape) != (T, Hq, Ev) or tuple(q.shape) != (F, T, Hq, E) or tuple(locations.shape) != (F, T):
+                raise ValueError("variable-length layout: q [F,T,Hq,E], locations [F,T], out [T,Hq,Ev]")
+            if tuple(fragment_lengths.shape) != (F, W) or tuple(cu_seqlens_q.shape) != (W + 1,):
+                raise ValueError("variable-length layout: fragment_lengths [F,W], cu_seqlens_q [W+1]")
+            lse_shape = (T, Hq)
+        else:
+            if out.dim() != 4 or out.size(0) != W:
+                raise ValueError("out must be [W, Hq, S, Ev] with one block-table row per worker")
+            _, Hq, S, _ = out.shape
+            T = 0
+            if tuple(out.shape) != (W, Hq, S, Ev) or tuple(q.shape) != (F, W, Hq, S, E) or tuple(locations.shape) != (F, W, S):
+                raise ValueError("fixed-length layout: q [F,W,Hq,S,E], locations [F,W,S], out [W,Hq,S,Ev]")
+            if tuple(fragment_lengths.shape) != (F,):
+                raise ValueError("fixed-length layout: fragment_lengths [F]")
+            lse_shape = (W, Hq, S)
+        tensors = [out, q, locations, fragment_lengths, key_cache, value_cache, block_table]
+        if varlen:
+            tensors.append(cu_seqlens_q)
+        if lse is not None:
+            if tuple(lse.shape) != lse_shape or lse.dtype != torch.float32:
+                raise ValueError(f"lse must be float32 {lse_shape}")
+            tensors.append(lse)
+        for t in (locations, fragment_lengths, block_table) + ((cu_seqlens_q,) if varlen else ()):
+            if t.dtype != torch.int32:
+                raise ValueError("locations, fragment_lengths, block_table and cu_seqlens_q must be int32")
+        for t in (q, key_cache, value_cache):
+            if t.dtype != out.dtype:
+                raise ValueError("queries and caches must have the dtype of the output")
+        for t in tensors:
+            if not t.is_contiguous():
+                raise ValueError("all tensors must be contiguous")
+            if t.device != out.device:
+                raise ValueError("all tensors must live on the output's device")
+        self._keep = tensors
+        self.device = out.device
+        p = HwPagedProblem()
+        p.dtype = _DTYPE_CODE[out.dtype]
+        p.F, p.W, p.Hq, p.Hkv, p.E, p.Ev, p.S, p.total_q = F, W, Hq, Hkv, E, Ev, S, T
+        p.block_size, p.max_blocks, p.num_blocks = BS, block_table.size(1), NB
+        p.scale = float(scale)
+        p.out = out.data_ptr()
+        p.lse = lse.data_ptr() if lse is not None else None
+        p.q = q.data_ptr()
+        p.locations = locations.data_ptr()
+        p.fragment_lengths = fragment_lengths.data_ptr()
+        p.key_cache = key_cache.data_ptr()
+        p.value_cache = value_cache.data_ptr()
+        p.block_table = block_table.data_ptr()
+        p.cu_seqlens_q = cu_seqlens_q.data_ptr() if varlen else None
+        p.splits = int(splits)
+        p.row_blocks = int(row_blocks)
+        self.p = p
+        self.varlen = varlen
+        self._ws = None
+
+    def workspace_bytes(self) -> int:
+        n = C.c_size_t(0)
+        with torch.cuda.device(self.device):
+            check(lib.hw_paged_workspace_bytes(C.byref(self.p), C.byref(n)), "hw_paged_workspace_bytes")
+        return n.value
+
+    def set_workspace(self, ws: Optional[torch.Tensor] = None) -> None:
+        if ws is None:
+            ws = torch.empty(max(self.workspace_bytes(), 256), dtype=torch.uint8, device=self.device)
+        self._ws = ws
+        self.p.workspace = ws.data_ptr()
+        self.p.workspace_bytes = ws.numel() * ws.element_size()
+
+    def run(self, stages: int = 3) -> None:
+        if self._ws is None:
+            self.set_workspace()
+        with torch.cuda.device(self.device):
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            if stages != 3:
+                check(lib.hw_paged_sdpa_stages(C.byref(self.p), C.c_void_p(stream), stages), "hw_paged_sdpa_stages")
+                return
+            fn = lib.hw_varlen_paged_sdpa if self.varlen else lib.hw_paged_sdpa
+            check(fn(C.byref(self.p), C.c_void_p(stream)), fn.__name__)
+
+
+def paged_plan(*, W: int, Hq: int, Hkv: int, Ev: int, block_size: int, max_blocks: int, num_cus: int, S: int = 0,
+               total_q: Optional[int] = None, splits: int = 0, dtype: int = HW_BF16, row_blocks: int = 0) -> HwPagedPlan:
+    """Host-only plan of the paged operators (no GPU needed); total_q selects the variable-length operator."""
+    p = HwPagedProblem()
+    p.dtype = dtype
+    p.F, p.W, p.Hq, p.Hkv, p.E, p.Ev, p.S = 1, W, Hq, Hkv, Ev, Ev, S
+    p.block_size, p.max_blocks, p.num_blocks = block_size, max_blocks, 1
+    if total_q is not None:
+        p.total_q = total_q
+        p.cu_seqlens_q = 16       # only tested for being non-NULL by the planner
+    p.splits = splits
+    p.row_blocks = row_blocks
+    out = HwPagedPlan()
+    check(lib.hw_paged_plan_debug(C.byref(p), num_cus, C.byref(out)), "hw_paged_plan_debug")
+    return out
+
+
+def copy_to_blocks(key_states: torch.Tensor, value_states: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                   block_table: torch.Tensor, seq_lengths: torch.Tensor) -> None:
+    """Append key_states / value_states [B, Hkv, S_new, E|Ev] (any strides with a contiguous last dimension) to the
+    paged caches at positions seq_lengths[b] + t."""
+    if key_states.dim() != 4 or value_states.dim() != 4 or key_states.shape[:3] != value_states.shape[:3]:
+        raise ValueError("key_states / value_states must be [B, Hkv, S_new, E|Ev]")
+    B, Hkv, S_new, E = key_states.shape
+    Ev = value_states.size(3)
+    if key_cache.dim() != 4 or value_cache.dim() != 4 or key_cache.size(1) != Hkv or key_cache.size(3) != E \
+            or value_cache.size(3) != Ev or key_cache.shape[:3] != value_cache.shape[:3]:
+        raise ValueError("caches must be [num_blocks, Hkv, block_size, E|Ev]")
+    if key_states.dtype not in _DTYPE_CODE:
+        raise HogwildError(-2, "copy_to_blocks")
+    for t in (value_states, key_cache, value_cache):
+        if t.dtype != key_states.dtype:
+            raise ValueError("states and caches must share one dtype")
+    if tuple(seq_lengths.shape) != (B,) or block_table.dim() != 2 or block_table.size(0) != B:
+        raise ValueError("block_table must be [B, max_blocks], seq_lengths [B]")
+    for t in (block_table, seq_lengths):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise ValueError("block_table and seq_lengths must be contiguous int32")
+    if not key_cache.is_contiguous() or not value_cache.is_contiguous():
+        raise ValueError("caches must be contiguous")
+    if (E > 1 and key_states.stride(3) != 1) or (Ev > 1 and value_states.stride(3) != 1):
+        key_states, value_states = key_states.contiguous(), value_states.contiguous()
+    for t in (key_states, value_states, value_cache, block_table, seq_lengths):
+        if t.device != key_cache.device:
+            raise ValueError("all tensors must live on the caches' device")
+    c = HwCopyBlocks()
+    c.dtype = _DTYPE_CODE[key_states.dtype]
+    c.B, c.Hkv, c.S_new, c.E, c.Ev = B, Hkv, S_new, E, Ev
+    c.block_size, c.max_blocks, c.num_blocks = key_cache.size(2), block_table.size(1), key_cache.size(0)
+    c.key_states, c.value_states = key_states.data_ptr(), value_states.data_ptr()
+    c.ks_b, c.ks_h, c.ks_s = key_states.stride(0), key_states.stride(1), key_states.stride(2)
+    c.vs_b, c.vs_h, c.vs_s = value_states.stride(0), value_states.stride(1), value_states.stride(2)
+    c.key_cache, c.value_cache = key_cache.data_ptr(), value_cache.data_ptr()
+    c.block_table, c.seq_lengths = block_table.data_ptr(), seq_lengths.data_ptr()
+    with torch.cuda.device(key_cache.device):
+        stream = torch.cuda.current_stream(key_cache.device).cuda_stream
+        check(lib.hw_copy_to_blocks(C.byref(c), C.c_void_p(stream)), "hw_copy_to_blocks")
 
 
 def rope(q: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -1,7 +1,7 @@
 // PyTorch operator binding for the MI355X Hogwild! attention library.
 //
-// Registers the operators of the reference's namespace `libhogatt` that lie on the fused decode path, with
-// the same schema strings (src/binding.cu:363-367 of the reference), on the dispatch key ROCm tensors use
+// Registers the operators of the reference's namespace `libhogatt` (the fused decode path and its paged
+// variants), with the same schema strings (src/binding.cu:363-374 of the reference), on the dispatch key ROCm tensors use
 // (CUDA).  Every operator only unpacks tensors into the plain-pointer hw_problem of include/hogwild_hip.h and
 // calls the C ABI on the current HIP stream; no device code lives here.
 //
@@ -222,6 +222,130 @@ void hogwild_fused_lse(at::Tensor& out, at::Tensor& rq, at::Tensor& lse, double 
     run(u, out, true);
 }
 
+// ---- paged operators -------------------------------------------------------------------------------------------
+
+// Checks shared by the two paged attention operators; fills everything of hw_paged_problem except the query layout.
+void unpack_paged(hw_paged_problem& p, at::Tensor& out, double scale, const at::Tensor& locations, const at::Tensor& queries,
+                  const at::Tensor& fragment_lengths, const at::Tensor& key_cache, const at::Tensor& value_cache,
+                  const at::Tensor& block_table) {
+    TORCH_CHECK(key_cache.dim() == 4 && value_cache.dim() == 4, "libhogatt: caches must be [num_blocks, Hkv, block_size, D]");
+    TORCH_CHECK(key_cache.size(0) == value_cache.size(0) && key_cache.size(1) == value_cache.size(1) && key_cache.size(2) == value_cache.size(2),
+                "libhogatt: key_cache and value_cache differ in blocks, heads or block size");
+    TORCH_CHECK(block_table.dim() == 2 && block_table.scalar_type() == at::kInt && block_table.is_contiguous(),
+                "libhogatt: block_table must be contiguous int32 [W, max_blocks]");
+    TORCH_CHECK(locations.scalar_type() == at::kInt && locations.is_contiguous(), "libhogatt: locations must be contiguous int32");
+    TORCH_CHECK(fragment_lengths.scalar_type() == at::kInt && fragment_lengths.is_contiguous(), "libhogatt: fragment_lengths must be contiguous int32");
+    TORCH_CHECK(out.is_contiguous() && queries.is_contiguous() && key_cache.is_contiguous() && value_cache.is_contiguous(),
+                "libhogatt: output, queries and caches must be contiguous");
+    TORCH_CHECK(queries.scalar_type() == out.scalar_type() && key_cache.scalar_type() == out.scalar_type() && value_cache.scalar_type() == out.scalar_type(),
+                "libhogatt: queries and caches must have the dtype of the output");
+    for (const at::Tensor* t : {&locations, &queries, &fragment_lengths, &key_cache, &value_cache, &block_table})
+        TORCH_CHECK(t->device() == out.device(), "libhogatt: all tensors must live on the output's device");
+    p.dtype = dtype_code(out);
+    p.F = (int32_t)locations.size(0);
+    p.W = (int32_t)block_table.size(0);
+    p.Hkv = (int32_t)key_cache.size(1);
+    p.E = (int32_t)key_cache.size(3);
+    p.Ev = (int32_t)value_cache.size(3);
+    p.block_size = (int32_t)key_cache.size(2);
+    p.max_blocks = (int32_t)block_table.size(1);
+    p.num_blocks = (int32_t)key_cache.size(0);
+    p.scale = (float)scale;
+    p.out = out.data_ptr();
+    p.q = queries.const_data_ptr();
+    p.locations = locations.const_data_ptr<int32_t>();
+    p.fragment_lengths = fragment_lengths.const_data_ptr<int32_t>();
+    p.key_cache = key_cache.const_data_ptr();
+    p.value_cache = value_cache.const_data_ptr();
+    p.block_table = block_table.const_data_ptr<int32_t>();
+}
+
+void run_paged(hw_paged_problem& p, const at::Tensor& out, bool varlen) {
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(out.device());
+    size_t bytes = 0;
+    check_status(hw_paged_workspace_bytes(&p, &bytes), "hw_paged_workspace_bytes");
+    at::Tensor workspace = at::empty({(int64_t)(bytes > 0 ? bytes : 256)}, out.options().dtype(at::kByte));
+    p.workspace = workspace.data_ptr();
+    p.workspace_bytes = bytes;
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(out.device().index()).stream();
+    if (varlen)
+        check_status(hw_varlen_paged_sdpa(&p, stream), "hw_varlen_paged_sdpa");
+    else
+        check_status(hw_paged_sdpa(&p, stream), "hw_paged_sdpa");
+}
+
+void hogwild_paged_sdpa(at::Tensor& out, double scale, const at::Tensor& locations, const at::Tensor& queries,
+                        const at::Tensor& fragment_lengths, const at::Tensor& key_cache, const at::Tensor& value_cache,
+                        const at::Tensor& block_table) {
+    hw_paged_problem p{};
+    unpack_paged(p, out, scale, locations, queries, fragment_lengths, key_cache, value_cache, block_table);
+    TORCH_CHECK(out.dim() == 4 && out.size(0) == p.W && out.size(3) == p.Ev, "libhogatt: output must be [W, Hq, S, Ev] with one block-table row per worker");
+    p.Hq = (int32_t)out.size(1);
+    p.S = (int32_t)out.size(2);
+    TORCH_CHECK(queries.dim() == 5 && queries.size(0) == p.F && queries.size(1) == p.W && queries.size(2) == p.Hq && queries.size(3) == p.S && queries.size(4) == p.E,
+                "libhogatt: queries must be [F, W, Hq, S, E]");
+    TORCH_CHECK(locations.dim() == 3 && locations.size(1) == p.W && locations.size(2) == p.S, "libhogatt: locations must be [F, W, S]");
+    TORCH_CHECK(fragment_lengths.dim() == 1 && fragment_lengths.size(0) == p.F, "libhogatt: fragment_lengths must be [F]");
+    run_paged(p, out, false);
+}
+
+void hogwild_varlen_paged_sdpa(at::Tensor& out, double scale, const at::Tensor& locations, const at::Tensor& queries,
+                               const at::Tensor& fragment_lengths, const at::Tensor& key_cache, const at::Tensor& value_cache,
+                               const at::Tensor& block_table, const at::Tensor& cu_seqlens_q, const at::Tensor& cu_seqlens_k) {
+    hw_paged_problem p{};
+    unpack_paged(p, out, scale, locations, queries, fragment_lengths, key_cache, value_cache, block_table);
+    TORCH_CHECK(out.dim() == 3 && out.size(2) == p.Ev, "libhogatt: output must be [total_q, Hq, Ev]");
+    p.total_q = (int32_t)out.size(0);
+    p.Hq = (int32_t)out.size(1);
+    TORCH_CHECK(queries.dim() == 4 && queries.size(0) == p.F && queries.size(1) == p.total_q && queries.size(2) == p.Hq && queries.size(3) == p.E,
+                "libhogatt: queries must be [F, total_q, Hq, E]");
+    TORCH_CHECK(locations.dim() == 2 && locations.size(1) == p.total_q, "libhogatt: locations must be [F, total_q]");
+    TORCH_CHECK(fragment_lengths.dim() == 2 && fragment_lengths.size(0) == p.F && fragment_lengths.size(1) == p.W,
+                "libhogatt: fragment_lengths must be [F, W]");
+    TORCH_CHECK(cu_seqlens_q.dim() == 1 && cu_seqlens_q.size(0) == p.W + 1 && cu_seqlens_q.scalar_type() == at::kInt &&
+                    cu_seqlens_q.is_contiguous() && cu_seqlens_q.device() == out.device(),
+                "libhogatt: cu_seqlens_q must be contiguous int32 [W + 1] on the output's device");
+    (void)cu_seqlens_k;   // carried in the reference's Shape but never read by its kernel (src/kernels/kernel_v21.cuh:658-899)
+    p.cu_seqlens_q = cu_seqlens_q.const_data_ptr<int32_t>();
+    run_paged(p, out, true);
+}
+
+void copy_to_blocks(const at::Tensor& key_states, const at::Tensor& value_states, at::Tensor& key_cache, at::Tensor& value_cache,
+                    const at::Tensor& block_table, const at::Tensor& seq_lengths) {
+    TORCH_CHECK(key_states.dim() == 4 && value_states.dim() == 4, "libhogatt: key_states / value_states must be [B, Hkv, S_new, D]");
+    TORCH_CHECK(key_states.size(0) == value_states.size(0) && key_states.size(1) == value_states.size(1) && key_states.size(2) == value_states.size(2),
+                "libhogatt: key_states and value_states differ in batch, heads or tokens");
+    TORCH_CHECK(key_cache.dim() == 4 && value_cache.dim() == 4 && key_cache.is_contiguous() && value_cache.is_contiguous(),
+                "libhogatt: caches must be contiguous [num_blocks, Hkv, block_size, D]");
+    TORCH_CHECK(key_cache.size(0) == value_cache.size(0) && key_cache.size(1) == key_states.size(1) && value_cache.size(1) == key_states.size(1) &&
+                    key_cache.size(2) == value_cache.size(2) && key_cache.size(3) == key_states.size(3) && value_cache.size(3) == value_states.size(3),
+                "libhogatt: caches do not match the states");
+    TORCH_CHECK(value_states.scalar_type() == key_states.scalar_type() && key_cache.scalar_type() == key_states.scalar_type() &&
+                    value_cache.scalar_type() == key_states.scalar_type(), "libhogatt: states and caches must share one dtype");
+    TORCH_CHECK(block_table.dim() == 2 && block_table.size(0) == key_states.size(0) && block_table.scalar_type() == at::kInt && block_table.is_contiguous(),
+                "libhogatt: block_table must be contiguous int32 [B, max_blocks]");
+    TORCH_CHECK(seq_lengths.dim() == 1 && seq_lengths.size(0) == key_states.size(0) && seq_lengths.scalar_type() == at::kInt && seq_lengths.is_contiguous(),
+                "libhogatt: seq_lengths must be contiguous int32 [B]");
+    for (const at::Tensor* t : std::initializer_list<const at::Tensor*>{&key_states, &value_states, &value_cache, &block_table, &seq_lengths})
+        TORCH_CHECK(t->device() == key_cache.device(), "libhogatt: all tensors must live on the caches' device");
+    // any strides are fine as long as the head dimension is contiguous (the transposed view of a projection is)
+    const at::Tensor ks = (key_states.size(3) > 1 && key_states.stride(3) != 1) ? key_states.contiguous() : key_states;
+    const at::Tensor vs = (value_states.size(3) > 1 && value_states.stride(3) != 1) ? value_states.contiguous() : value_states;
+    hw_copy_blocks c{};
+    c.dtype = dtype_code(key_states);
+    c.B = (int32_t)ks.size(0); c.Hkv = (int32_t)ks.size(1); c.S_new = (int32_t)ks.size(2);
+    c.E = (int32_t)ks.size(3); c.Ev = (int32_t)vs.size(3);
+    c.block_size = (int32_t)key_cache.size(2); c.max_blocks = (int32_t)block_table.size(1); c.num_blocks = (int32_t)key_cache.size(0);
+    c.key_states = ks.const_data_ptr(); c.value_states = vs.const_data_ptr();
+    c.ks_b = ks.stride(0); c.ks_h = ks.stride(1); c.ks_s = ks.stride(2);
+    c.vs_b = vs.stride(0); c.vs_h = vs.stride(1); c.vs_s = vs.stride(2);
+    c.key_cache = key_cache.data_ptr(); c.value_cache = value_cache.data_ptr();
+    c.block_table = block_table.const_data_ptr<int32_t>(); c.seq_lengths = seq_lengths.const_data_ptr<int32_t>();
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(key_cache.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(key_cache.device().index()).stream();
+    check_status(hw_copy_to_blocks(&c, stream), "hw_copy_to_blocks");
+}
+
 }  // namespace
 
 // `import hogatt` only has to load this shared object so that the registrations below run.
@@ -242,6 +366,13 @@ TORCH_LIBRARY(libhogatt, m) {
           "Tensor fragment_lengths, Tensor[] key_fragments, Tensor[] value_fragments) -> ()", tags);
     m.def("hogwild_fused_lse(Tensor(a!) output, Tensor(b!) rq, Tensor(c!) lse, float scale, Tensor locations, Tensor queries, "
           "Tensor fragment_lengths, Tensor[] key_fragments, Tensor[] value_fragments, Tensor cosines, Tensor sines) -> ()", tags);
+    // the paged operators, schemas of src/binding.cu:369-374
+    m.def("hogwild_paged_sdpa(Tensor(a!) output, float scale, Tensor locations, Tensor queries, "
+          "Tensor fragment_lengths, Tensor key_cache, Tensor value_cache, Tensor block_table) -> ()", tags);
+    m.def("copy_to_blocks(Tensor key_states, Tensor value_states, Tensor(a!) key_cache, Tensor(b!) value_cache, "
+          "Tensor block_table, Tensor seq_lengths) -> ()", tags);
+    m.def("hogwild_varlen_paged_sdpa(Tensor(a!) output, float scale, Tensor locations, Tensor queries, "
+          "Tensor fragment_lengths, Tensor key_cache, Tensor value_cache, Tensor block_table, Tensor cu_seqlens_q, Tensor cu_seqlens_k) -> ()", tags);
 }
 
 TORCH_LIBRARY_IMPL(libhogatt, CUDA, m) {
@@ -250,4 +381,7 @@ TORCH_LIBRARY_IMPL(libhogatt, CUDA, m) {
     m.impl("hogwild_fused", hogwild_fused);
     m.impl("hogwild_sdpa_lse", hogwild_sdpa_lse);
     m.impl("hogwild_fused_lse", hogwild_fused_lse);
+    m.impl("hogwild_paged_sdpa", hogwild_paged_sdpa);
+    m.impl("copy_to_blocks", copy_to_blocks);
+    m.impl("hogwild_varlen_paged_sdpa", hogwild_varlen_paged_sdpa);
 }

@@ -241,6 +241,156 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     return (int)e;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// paged variants
+// ---------------------------------------------------------------------------------------------------------
+int paged_validate(const hw_paged_problem* p) {
+    if (p == nullptr) return HW_ERR_NULL;
+    if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
+    if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
+    if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return HW_ERR_SHAPE;
+    const bool varlen = p->cu_seqlens_q != nullptr;
+    if (varlen ? p->total_q < 0 : (p->S < 1 || p->S >= (1 << 12))) return HW_ERR_SHAPE;
+    if (p->block_size < 1 || p->block_size >= (1 << 12) || p->max_blocks < 1 || p->num_blocks < 1) return HW_ERR_SHAPE;
+    if ((long long)p->block_size * p->max_blocks > (1ll << 20)) return HW_ERR_SHAPE;
+    if ((long long)p->num_blocks * p->Hkv * p->block_size >= (1ll << 31)) return HW_ERR_SHAPE;
+    const long long tokens = varlen ? p->total_q : (long long)p->W * p->S;
+    const int gq = p->Hq / p->Hkv;
+    if (gq >= (1 << 12) || tokens * gq >= (1 << 20) || p->W >= (1 << 20)) return HW_ERR_SHAPE;
+    if (p->out == nullptr || p->q == nullptr || p->locations == nullptr || p->fragment_lengths == nullptr) {
+        if (tokens > 0) return HW_ERR_NULL;
+    }
+    if (p->key_cache == nullptr || p->value_cache == nullptr || p->block_table == nullptr) return HW_ERR_NULL;
+    if (!aligned16(p->out) || !aligned16(p->q) || !aligned16(p->key_cache) || !aligned16(p->value_cache)) return HW_ERR_ALIGN;
+    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
+    return HW_OK;
+}
+
+int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
+    if (plan == nullptr) return HW_ERR_NULL;
+    if (num_cus < 1) return HW_ERR_SHAPE;
+    std::memset(plan, 0, sizeof(*plan));
+    const bool varlen = p->cu_seqlens_q != nullptr;
+    const int gq = p->Hq / p->Hkv;
+    const long long tokens = varlen ? p->total_q : (long long)p->W * p->S;
+    plan->rows = (int)(tokens * gq);
+    // rows of one worker share its KV: one 16-row block is enough for plain decoding, two when a worker brings
+    // more rows (several query tokens, wide GQA groups)
+    const long long rows_per_worker = varlen ? (tokens * gq + p->W - 1) / p->W : (long long)p->S * gq;
+    plan->row_blocks = rows_per_worker <= 16 ? 1 : 2;
+    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
+    if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
+    const int rpw = 16 * plan->row_blocks;
+    long long items;
+    if (varlen) items = p->W + tokens * gq / rpw;          // sum_w ceil(rows_w / rpw) <= W + rows / rpw
+    else items = (long long)p->W * (((long long)p->S * gq + rpw - 1) / rpw);
+    if (items < 1) items = 1;
+    plan->row_groups = (int)items;
+    int splits = p->splits;
+    if (splits <= 0) {
+        const long long target = num_cus;   // the paged kernels are built for one workgroup per CU
+        long long s = target / ((long long)p->Hkv * items);
+        // at the longest sequence the table allows, every wave should still have at least one tile
+        const long long by_work = ((long long)p->block_size * p->max_blocks + hw::TILE * hw::NWAVES - 1) / (hw::TILE * hw::NWAVES);
+        if (s > by_work) s = by_work;
+        splits = (int)s;
+    }
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    plan->splits = splits;
+    const long long wgs = (long long)p->Hkv * items * splits;
+    if (wgs >= (1 << 20)) return HW_ERR_SHAPE;
+    plan->workgroups = (int)wgs;
+    plan->workspace_bytes = (size_t)p->Hkv * splits * (size_t)(plan->rows > 0 ? plan->rows : 1) * ((size_t)p->Ev + 2) * sizeof(float);
+    plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
+    return HW_OK;
+}
+
+int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
+    int st = paged_validate(p);
+    if (st != HW_OK) return st;
+    int cus = 0;
+    st = device_cus(&cus);
+    if (st != HW_OK) return st;
+    hw_paged_plan plan;
+    st = paged_plan(p, cus, &plan);
+    if (st != HW_OK) return st;
+    if (plan.rows == 0) return HW_OK;       // no query tokens
+    if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
+    hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
+    const bool varlen = p->cu_seqlens_q != nullptr;
+    auto magic = [](int d) { return (unsigned)(((1ull << 32) + (unsigned long long)d - 1) / (unsigned long long)d); };
+
+    hw::PagedHeader ph;
+    std::memset(&ph, 0, sizeof(ph));
+    ph.q = p->q;
+    ph.loc = p->locations;
+    ph.frag_len = p->fragment_lengths;
+    ph.kcache = p->key_cache;
+    ph.vcache = p->value_cache;
+    ph.block_table = p->block_table;
+    ph.cu_q = p->cu_seqlens_q;
+    ph.part_o = reinterpret_cast<float*>(p->workspace);
+    ph.part_ml = ph.part_o + (size_t)p->Hkv * plan.splits * plan.rows * p->Ev;
+    ph.F = p->F; ph.W = p->W; ph.Hq = p->Hq; ph.Hkv = p->Hkv;
+    ph.LW = varlen ? p->total_q : p->W;
+    ph.LS = varlen ? 1 : p->S;
+    ph.R = plan.rows;
+    ph.block_size = p->block_size; ph.max_blocks = p->max_blocks; ph.num_blocks = p->num_blocks;
+    ph.nsplit = plan.splits;
+    ph.nitems = plan.row_groups;
+    ph.nrg = varlen ? 1 : plan.row_groups / p->W;
+    ph.nwg = plan.workgroups;
+    ph.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
+    ph.sc = (float)((double)p->scale * 1.4426950408889634074);
+    ph.magic_gq = magic(p->Hq / p->Hkv);
+    ph.magic_ls = magic(ph.LS);
+    ph.magic_bs = magic(p->block_size);
+    ph.magic_nsplit = magic(ph.nsplit);
+    ph.magic_nitems = magic(ph.nitems);
+    ph.magic_nrg = magic(ph.nrg);
+
+    hipError_t e = hipSuccess;
+    if (stages & HW_STAGE_ATTENTION) {
+        e = hw::launch_paged_attention(ph, p->dtype, p->E, plan.row_blocks, stream);
+        if (e != hipSuccess) return (int)e;
+    }
+    if (!(stages & HW_STAGE_MERGE)) return (int)e;
+    hw::MergeArgs ma;
+    ma.part_o = ph.part_o;
+    ma.part_ml = ph.part_ml;
+    ma.out = p->out;
+    ma.lse = p->lse;
+    ma.W = ph.LW; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = ph.LS; ma.R = plan.rows;
+    ma.wgs_per_head = plan.splits;
+    // a variable-length launch may leave row groups of the grid unused, and with them parts of an XCD's share
+    ma.xcd_local = (!varlen && plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
+    e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
+    return (int)e;
+}
+
+int copy_blocks_run(const hw_copy_blocks* c, void* stream) {
+    if (c == nullptr) return HW_ERR_NULL;
+    if (c->dtype != HW_F32 && c->dtype != HW_F16 && c->dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (c->B < 0 || c->Hkv < 1 || c->S_new < 0 || c->E < 1 || c->Ev < 1) return HW_ERR_SHAPE;
+    if (c->block_size < 1 || c->max_blocks < 1 || c->num_blocks < 1) return HW_ERR_SHAPE;
+    if ((long long)c->num_blocks * c->Hkv * c->block_size >= (1ll << 31)) return HW_ERR_SHAPE;
+    if (c->B == 0 || c->S_new == 0) return HW_OK;
+    if (c->key_states == nullptr || c->value_states == nullptr || c->key_cache == nullptr || c->value_cache == nullptr ||
+        c->block_table == nullptr || c->seq_lengths == nullptr)
+        return HW_ERR_NULL;
+    hw::CopyBlocksArgs a;
+    a.key_states = c->key_states; a.value_states = c->value_states;
+    a.kcache = c->key_cache; a.vcache = c->value_cache;
+    a.block_table = c->block_table; a.seq_lengths = c->seq_lengths;
+    a.ks_b = c->ks_b; a.ks_h = c->ks_h; a.ks_s = c->ks_s; a.vs_b = c->vs_b; a.vs_h = c->vs_h; a.vs_s = c->vs_s;
+    a.B = c->B; a.Hkv = c->Hkv; a.S_new = c->S_new; a.E = c->E; a.Ev = c->Ev;
+    a.block_size = c->block_size; a.max_blocks = c->max_blocks; a.num_blocks = c->num_blocks;
+    return (int)hw::launch_copy_to_blocks(a, c->dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
 }  // namespace
 
 extern "C" {
@@ -306,6 +456,44 @@ int hw_rope(void* out, const void* q, const float* cosines, const float* sines, 
     if (RotE > 0 && (cosines == nullptr || sines == nullptr)) return HW_ERR_NULL;
     return (int)hw::launch_rope(out, q, cosines, sines, dtype, F, W, Hq, S, E, RotE, reinterpret_cast<hipStream_t>(stream));
 }
+
+int hw_paged_validate(const hw_paged_problem* p) { return paged_validate(p); }
+
+int hw_paged_plan_debug(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
+    if (p == nullptr || plan == nullptr) return HW_ERR_NULL;
+    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->Ev < 1 || p->Hq % p->Hkv != 0 || p->block_size < 1 || p->max_blocks < 1) return HW_ERR_SHAPE;
+    if (p->cu_seqlens_q != nullptr ? p->total_q < 0 : p->S < 1) return HW_ERR_SHAPE;
+    return paged_plan(p, num_cus, plan);
+}
+
+int hw_paged_workspace_bytes(const hw_paged_problem* p, size_t* bytes) {
+    if (bytes == nullptr) return HW_ERR_NULL;
+    int cus = 0;
+    int st = device_cus(&cus);
+    if (st != HW_OK) return st;
+    hw_paged_plan plan;
+    st = hw_paged_plan_debug(p, cus, &plan);
+    if (st != HW_OK) return st;
+    *bytes = plan.workspace_bytes;
+    return HW_OK;
+}
+
+int hw_paged_sdpa(const hw_paged_problem* p, void* stream) {
+    if (p != nullptr && p->cu_seqlens_q != nullptr) return HW_ERR_SHAPE;
+    return paged_run(p, stream, HW_STAGE_ATTENTION | HW_STAGE_MERGE);
+}
+
+int hw_varlen_paged_sdpa(const hw_paged_problem* p, void* stream) {
+    if (p != nullptr && p->cu_seqlens_q == nullptr) return HW_ERR_NULL;
+    return paged_run(p, stream, HW_STAGE_ATTENTION | HW_STAGE_MERGE);
+}
+
+int hw_paged_sdpa_stages(const hw_paged_problem* p, void* stream, int stages) {
+    if ((stages & (HW_STAGE_ATTENTION | HW_STAGE_MERGE)) == 0 || (stages & ~(HW_STAGE_ATTENTION | HW_STAGE_MERGE)) != 0) return HW_ERR_SHAPE;
+    return paged_run(p, stream, stages);
+}
+
+int hw_copy_to_blocks(const hw_copy_blocks* c, void* stream) { return copy_blocks_run(c, stream); }
 
 int hw_device_cus(void) {
     int c = 0;

@@ -1,0 +1,561 @@
+// Device-side building blocks shared by the attention kernels of this library (gfx950, wave64): element traits,
+// tile geometry, K/V tile loads, the per-tile MFMA + online-softmax step, query staging.  Included by the .hip
+// translation units only.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hogwild_kernels.h"
+
+#ifndef HW_MARK
+#define HW_MARK(i) do { } while (0)
+#endif
+
+namespace hw {
+
+typedef unsigned int u32;
+typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+typedef u32 u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+struct BF16 {};
+struct F16 {};
+struct F32 {};
+
+template <class DT> struct Elem;
+template <> struct Elem<BF16> {
+    typedef unsigned short store_t;
+    static constexpr int size = 2;
+    static __device__ __forceinline__ float to_float(store_t x) { return __uint_as_float(((u32)x) << 16); }
+    static __device__ __forceinline__ store_t from_float(float f) {
+        __bf16 h = (__bf16)f;
+        return __builtin_bit_cast(unsigned short, h);
+    }
+    static __device__ __forceinline__ u32 pack2(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2));
+    }
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Elem<F16> {
+    typedef unsigned short store_t;
+    static constexpr int size = 2;
+    static __device__ __forceinline__ float to_float(store_t x) { return (float)__builtin_bit_cast(_Float16, x); }
+    static __device__ __forceinline__ store_t from_float(float f) {
+        _Float16 h = (_Float16)f;
+        return __builtin_bit_cast(unsigned short, h);
+    }
+    static __device__ __forceinline__ u32 pack2(float a, float b) {
+        f32x2 v = {a, b};
+        return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2));
+    }
+    static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+template <> struct Elem<F32> {
+    typedef float store_t;
+    static constexpr int size = 4;
+    static __device__ __forceinline__ float to_float(store_t x) { return x; }
+    static __device__ __forceinline__ store_t from_float(float f) { return f; }
+};
+
+constexpr float NEG_BIG = -1.0e30f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// max over the four lanes {l, l^16, l^32, l^48}: the four quarter-waves hold different tokens of one row
+__device__ __forceinline__ float quarter_max(float v) {
+    v = fmaxf(v, __shfl_xor(v, 16, 64));
+    v = fmaxf(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+__device__ __forceinline__ float quarter_sum(float v) {
+    v += __shfl_xor(v, 16, 64);
+    v += __shfl_xor(v, 32, 64);
+    return v;
+}
+
+// token (relative to the tile start) held in reduction slot `idx` (0..7) of quarter-wave `q`:
+// slots 0..3 come from the first 16-token S^T block, 4..7 from the second (accumulator rows 4q..4q+3).
+__device__ __forceinline__ int slot_token(int q, int idx) { return ((idx >> 2) << 4) + (q << 2) + (idx & 3); }
+
+template <class DT, int E, int EV>
+struct Geo {
+    static constexpr int SZ = Elem<DT>::size;
+    static constexpr int KJ = E * SZ / 64;               // 16-byte K operand chunks per lane per 16-token block
+    static constexpr int KROW = E * SZ;                  // bytes of one K row
+    static constexpr int VROW = EV * SZ;                 // bytes of one V row
+    static constexpr int CPR = KROW / 16;                // 16-byte chunks per K row
+    static constexpr int KL = TILE * KROW / 1024;        // 1 KB wave-wide K loads per tile
+    static constexpr int KSTAGE = TILE * KROW;           // bytes of the per-wave K staging area in LDS
+    static constexpr int VW = EV * SZ / 64;              // dwords of one V row held by one lane
+    static constexpr int VLD = VW < 4 ? VW : 4;          // dwords per V load
+    static constexpr int NVL = VW / VLD;                 // V loads per row per lane
+    static constexpr int NOC = EV / 16;                  // 16-wide output chunks (accumulators per row block)
+    static constexpr int QSTR = E * SZ + 16;             // LDS row stride of the rotated query (bytes)
+};
+
+// Registers of one 32-token tile of one wave: only V lives in registers, K goes straight from global memory
+// into the wave's LDS staging slot.
+template <class DT, int E, int EV>
+struct TileRegs {
+    typedef Geo<DT, E, EV> G;
+    u32 v[8][G::VW];     // V rows of the lane's 8 reduction slots, VW dwords of each
+};
+
+#define HW_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+
+// A fragment's K and V slices of one kv head as buffer resources: out-of-range rows read as zero, so tiles
+// need no address clamping, and a tile that does not exist costs no memory traffic at all.
+struct FragView {
+    __amdgpu_buffer_rsrc_t k, v;
+};
+constexpr unsigned OOB_OFFSET = 0xFFFF0000u;   // beyond any fragment (lengths are validated on the host)
+
+__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int krow, int vrow) {
+    FragView fv;
+    fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * L * krow), 0, L * krow, 0x00020000);
+    fv.v = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(vptr + (unsigned long long)hkv * L * vrow), 0, L * vrow, 0x00020000);
+    return fv;
+}
+
+// LDS position of 16-byte chunk c of tile row `row` in a K staging slot.  The xor key makes the operand read
+// (16 lanes = 16 different rows, same chunk) touch 16 different 16-byte bank groups.
+template <class G>
+__device__ __forceinline__ int kstage_offset(int row, int c) {
+    const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+    return row * G::KROW + ((c ^ key) << 4);
+}
+
+// Per-lane byte offsets (within a tile) of the K chunk each lane fetches in each of the KL wave-wide loads.
+// A load writes LDS linearly (lane l -> slot base + 16 l), so the bank swizzle of kstage_offset is applied on
+// the global side: the lane that fills position (row, slot) fetches chunk slot ^ key(row) of that row.  The 16
+// lanes of a row still cover the row's bytes exactly once, so every load remains 1 KB of whole rows.
+template <class G>
+__device__ __forceinline__ void k_lane_offsets(unsigned* koff, int lane) {
+#pragma unroll
+    for (int i = 0; i < G::KL; ++i) {
+        const int p = i * 64 + lane;
+        const int row = p / G::CPR, slot = p % G::CPR;
+        const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+        koff[i] = row * G::KROW + ((slot ^ key) << 4);
+    }
+}
+
+// Issue the loads of one tile: K by direct global->LDS transfers into `kslot` (this wave's part of a staging
+// slot), V into registers.  The number of load instructions is the same whether or not the tile exists, which
+// keeps the hardware wait counts exact on every path; a tile that does not exist reads out of range (zeros,
+// no memory traffic).
+template <class DT, int E, int EV>
+__device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView& fv, char* kslot, const unsigned* koff, int t0,
+                                          int n, int q, bool real) {
+    typedef Geo<DT, E, EV> G;
+    const unsigned kb = real ? (unsigned)(t0 * G::KROW) : OOB_OFFSET;
+#pragma unroll
+    for (int i = 0; i < G::KL; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, 0);
+    // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load
+    const unsigned vb = real ? (unsigned)((t0 + q * 4) * G::VROW + n * (G::VLD * 4)) : OOB_OFFSET;
+#pragma unroll
+    for (int idx = 0; idx < 8; ++idx) {
+        const int rowoff = ((idx >> 2) * 16 + (idx & 3)) * G::VROW;
+#pragma unroll
+        for (int hh = 0; hh < G::NVL; ++hh) {
+            if constexpr (G::VLD == 4) {
+                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(fv.v, vb + rowoff + hh * 256, 0, 0);
+                t.v[idx][hh * 4 + 0] = x.x;
+                t.v[idx][hh * 4 + 1] = x.y;
+                t.v[idx][hh * 4 + 2] = x.z;
+                t.v[idx][hh * 4 + 3] = x.w;
+            } else {
+                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(fv.v, vb + rowoff, 0, 0);
+                t.v[idx][0] = x.x;
+                t.v[idx][1] = x.y;
+            }
+        }
+    }
+}
+
+// Running state of one wave: RB row blocks of 16 rows each.
+template <int RB, int NOC>
+struct WaveState {
+    f32x4 o[RB][NOC];
+    float m[RB];   // reference of the exponentials (base-2 units): within 2^8 below/above the running max
+    float l[RB];   // lane-partial sum: this lane's quarter of the tokens
+    bool fresh;    // no tile accumulated yet (uniform over the wave)
+};
+
+// One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG>
+__device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
+                                             WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage) {
+    typedef Geo<DT, E, EV> G;
+#ifdef HW_NO_COMPUTE   // tuning aid: consume the tile without doing the arithmetic
+    {
+        u32 x = 0;
+#pragma unroll
+        for (int idx = 0; idx < 8; ++idx)
+#pragma unroll
+            for (int d = 0; d < G::VW; ++d) x ^= t.v[idx][d];
+        x ^= *reinterpret_cast<const u32*>(kstage + kstage_offset<G>(n, q));
+        st.l[0] += __uint_as_float(x & 0x3fffffffu);
+        return;
+    }
+#endif
+    // K operand: out of the staging slot in MFMA A-operand order (lane = token, 16 B of head dim).  The compiler
+    // tracks the outstanding global->LDS transfers per staging slot and waits for this slot's before the reads.
+    // S^T blocks: for each 16-token block, its K operand (lane = token, 16 B of head dim per k-step) against the
+    // B operand of every row block (this row's rotated query, from registers when QREG, else straight from LDS)
+    f32x4 sacc[RB][2];
+#pragma unroll
+    for (int tb = 0; tb < 2; ++tb) {
+        u32x4 kop[G::KJ];
+#pragma unroll
+        for (int j = 0; j < G::KJ; ++j) kop[j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            u32x4 qop[G::KJ];
+#pragma unroll
+            for (int j = 0; j < G::KJ; ++j)
+                qop[j] = QREG ? qreg[rb * G::KJ + j] : *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (G::SZ == 2) {
+#pragma unroll
+                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[j], qop[j], acc);
+            } else {
+#pragma unroll
+                for (int j = 0; j < G::KJ; ++j) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c)
+                        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(kop[j][c]), __uint_as_float(qop[j][c]), acc, 0, 0, 0);
+                }
+            }
+            sacc[rb][tb] = acc;
+        }
+    }
+    // Online softmax with a lazily updated reference: exponentials are taken against st.m, which only moves when
+    // a row's maximum exceeds it by more than 2^LAZY_LOG2 (then O and l of that row are rescaled).  Most tiles
+    // therefore leave the accumulators alone: no rescale multiplies, and O can stay in the MFMA accumulator
+    // registers.  p is at most 2^LAZY_LOG2, far inside the range of every storage type.
+    constexpr float LAZY_LOG2 = 8.0f;
+    float s[RB][8];
+    float mxs[RB];
+    bool need = false;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        float mx = NEG_BIG;
+#pragma unroll
+        for (int idx = 0; idx < 8; ++idx) {
+            s[rb][idx] = sacc[rb][idx >> 2][idx & 3];
+            if constexpr (MASKED) s[rb][idx] = (t0 + slot_token(q, idx)) < lim[rb] ? s[rb][idx] : NEG_BIG;
+            mx = fmaxf(mx, s[rb][idx]);
+        }
+        mx = quarter_max(mx);
+        mxs[rb] = mx < -1.0e29f ? NEG_BIG : mx * sc;      // sc > 0: scaling commutes with the max; nothing visible stays NEG_BIG
+        need = need || (mxs[rb] > st.m[rb] + LAZY_LOG2);
+    }
+    if (__builtin_amdgcn_ballot_w64(need) != 0) {        // uniform over the wave
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const float mnew = mxs[rb] > st.m[rb] + LAZY_LOG2 ? mxs[rb] : st.m[rb];
+            const float alpha = fast_exp2(st.m[rb] - mnew);   // 1 for rows that keep their reference
+            st.m[rb] = mnew;
+            st.l[rb] *= alpha;
+            if (!st.fresh) {                                  // before the first tile O is zero
+#pragma unroll
+                for (int c = 0; c < G::NOC; ++c) st.o[rb][c] *= alpha;
+            }
+        }
+    }
+    st.fresh = false;
+    float p[RB][8];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        // a row that has seen nothing yet keeps the reference NEG_BIG; exponentiate against 0 so its masked slots give 0
+        const float mref = MASKED ? (st.m[rb] < -1.0e29f ? 0.f : st.m[rb]) : st.m[rb];
+        float psum = 0.f;
+#pragma unroll
+        for (int idx = 0; idx < 8; ++idx) {
+            p[rb][idx] = fast_exp2(__builtin_fmaf(s[rb][idx], sc, -mref));
+            psum += p[rb][idx];
+        }
+        st.l[rb] += psum;
+    }
+
+    if constexpr (G::SZ == 2) {
+        u32x4 pp[RB];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            pp[rb].x = Elem<DT>::pack2(p[rb][0], p[rb][1]);
+            pp[rb].y = Elem<DT>::pack2(p[rb][2], p[rb][3]);
+            pp[rb].z = Elem<DT>::pack2(p[rb][4], p[rb][5]);
+            pp[rb].w = Elem<DT>::pack2(p[rb][6], p[rb][7]);
+        }
+        // dword d of a lane's V row holds ev (n*EVL + 2d, n*EVL + 2d + 1); gather the 8 tokens of each ev.
+#pragma unroll
+        for (int d = 0; d < G::VW; ++d) {
+            u32x4 lo, hi;
+            lo.x = __builtin_amdgcn_perm(t.v[1][d], t.v[0][d], 0x05040100u);
+            lo.y = __builtin_amdgcn_perm(t.v[3][d], t.v[2][d], 0x05040100u);
+            lo.z = __builtin_amdgcn_perm(t.v[5][d], t.v[4][d], 0x05040100u);
+            lo.w = __builtin_amdgcn_perm(t.v[7][d], t.v[6][d], 0x05040100u);
+            hi.x = __builtin_amdgcn_perm(t.v[1][d], t.v[0][d], 0x07060302u);
+            hi.y = __builtin_amdgcn_perm(t.v[3][d], t.v[2][d], 0x07060302u);
+            hi.z = __builtin_amdgcn_perm(t.v[5][d], t.v[4][d], 0x07060302u);
+            hi.w = __builtin_amdgcn_perm(t.v[7][d], t.v[6][d], 0x07060302u);
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                st.o[rb][2 * d] = Elem<DT>::mfma(lo, pp[rb], st.o[rb][2 * d]);
+                st.o[rb][2 * d + 1] = Elem<DT>::mfma(hi, pp[rb], st.o[rb][2 * d + 1]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int idx = 0; idx < 8; ++idx) {
+#pragma unroll
+            for (int c = 0; c < G::NOC; ++c) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+                    st.o[rb][c] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(t.v[idx][c]), p[rb][idx], st.o[rb][c], 0, 0, 0);
+            }
+        }
+    }
+}
+
+// head-dim index of accumulator chunk c, accumulator row i (0..15)
+template <class DT, int EV>
+__device__ __forceinline__ int out_ev(int c, int i) {
+    if constexpr (Elem<DT>::size == 2) {
+        return i * (EV / 16) + c;              // lane i of a V row holds EV/16 consecutive elements
+    } else {
+        return (c >> 2) * 64 + i * 4 + (c & 3);  // 16 lanes x 4 floats per 256-byte load, c>>2 selects the load
+    }
+}
+
+// 16-byte chunk of CH elements <-> CH floats
+template <class DT> struct Chunk;
+template <> struct Chunk<F32> {
+    static constexpr int CH = 4;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[4]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(x[i]);
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[4]) {
+        return u32x4{__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3])};
+    }
+};
+template <> struct Chunk<BF16> {
+    static constexpr int CH = 8;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[8]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f[2 * i] = __uint_as_float(x[i] << 16);
+            f[2 * i + 1] = __uint_as_float(x[i] & 0xffff0000u);
+        }
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        return u32x4{Elem<BF16>::pack2(f[0], f[1]), Elem<BF16>::pack2(f[2], f[3]), Elem<BF16>::pack2(f[4], f[5]),
+                     Elem<BF16>::pack2(f[6], f[7])};
+    }
+};
+template <> struct Chunk<F16> {
+    static constexpr int CH = 8;
+    static __device__ __forceinline__ void unpack(u32x4 x, float (&f)[8]) {
+        f16x8 h = __builtin_bit_cast(f16x8, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ u32x4 pack(const float (&f)[8]) {
+        return u32x4{Elem<F16>::pack2(f[0], f[1]), Elem<F16>::pack2(f[2], f[3]), Elem<F16>::pack2(f[4], f[5]),
+                     Elem<F16>::pack2(f[6], f[7])};
+    }
+};
+
+#define HW_GLOBAL __attribute__((address_space(1)))
+
+// What each wave of a workgroup hands over at the end (row stride padded so that rows land in different banks).
+template <int ROWS, int EV>
+struct Exchange {
+    float o[NWAVES][ROWS][EV + 4];
+    float m[NWAVES][ROWS];
+    float l[NWAVES][ROWS];
+};
+
+// Epilogue shared by the attention kernels: every wave hands over its raw accumulators, running max and sum
+// through LDS (one barrier); then all threads combine them with the weights 2^(m_wave - m_max) and store the
+// workgroup's partial coalesced: `nrows` rows starting at partial row index `part` (EV floats per row in part_o,
+// a (max, sum) pair per row in part_ml).  `ex` may alias a K staging slot: the leading barrier makes sure every
+// wave is done with it.
+template <class DT, int EV, int RB>
+__device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Exchange<RB * 16, EV>& ex, int wv, int n, int q, int tid,
+                                               HW_GLOBAL float* part_o, HW_GLOBAL float* part_ml, size_t part, int nrows) {
+    constexpr int NOC = EV / 16;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) st.l[rb] = quarter_sum(st.l[rb]);
+    // a look-ahead transfer into a staging slot may still be in flight; it must have landed before ANY wave writes `ex`
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int c = 0; c < NOC; ++c) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ex.o[wv][rb * 16 + n][out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
+        }
+        if (q == 0) {
+            ex.m[wv][rb * 16 + n] = st.m[rb];
+            ex.l[wv][rb * 16 + n] = st.l[rb];
+        }
+    }
+    __syncthreads();
+    HW_MARK(4);
+    HW_GLOBAL float* dst = part_o + part * EV;
+    for (int idx = tid * 4; idx < nrows * EV; idx += NTHREADS * 4) {
+        const int rr = idx / EV, e = idx - rr * EV;
+        float mm = ex.m[0][rr];
+#pragma unroll
+        for (int w2 = 1; w2 < NWAVES; ++w2) mm = fmaxf(mm, ex.m[w2][rr]);
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        float lsum = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < NWAVES; ++w2) {
+            const float wgt = fast_exp2(ex.m[w2][rr] - mm);
+            acc += *reinterpret_cast<const f32x4*>(&ex.o[w2][rr][e]) * wgt;
+            lsum += ex.l[w2][rr] * wgt;
+        }
+        *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = acc;
+        if (e == 0) {
+            HW_GLOBAL float* ml = part_ml + (part + rr) * 2;
+            ml[0] = mm;
+            ml[1] = lsum;
+        }
+    }
+}
+
+
+// KernelHeader as the kernel sees it after fetching it by hand: same layout, pointers typed as global memory
+// (a pointer rebuilt from raw bits would otherwise be a flat pointer, and flat loads tie up both wait counters).
+struct DevHeader {
+    const HW_GLOBAL char* q;
+    const HW_GLOBAL int* loc;
+    const HW_GLOBAL float* cos;
+    const HW_GLOBAL float* sin;
+    HW_GLOBAL char* rq;
+    HW_GLOBAL float* part_o;
+    HW_GLOBAL float* part_ml;
+    int F, W, Hq, Hkv, S, RotE, R;
+    int nrg, wgs_per_head, tiles_per_head, nwg;
+    int prerotated;
+    int xcd_remap;
+    float sc;
+    unsigned magic_gq, magic_s, magic_nrg, magic_wg;
+};
+static_assert(sizeof(DevHeader) == sizeof(KernelHeader), "DevHeader mirrors KernelHeader");
+
+// n / d for n < 2^20, d < 2^12 with the host-computed multiplier ceil(2^32 / d) mod 2^32: one multiply-high instead
+// of the ~25-instruction integer division sequence.  d == 1 gives the multiplier 0, which stands for "n itself".
+__device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
+
+// row r (0..R) of a kv head -> (worker*S + token, q head, flat q row index)
+struct RowMap {
+    int ws;
+    size_t qrow;
+};
+__device__ __forceinline__ RowMap map_row(const DevHeader& a, int r, int hkv, int GQ) {
+    RowMap m;
+    m.ws = fast_div(r, a.magic_gq);
+    const int gq = r - m.ws * GQ;
+    const int w = fast_div(m.ws, a.magic_s), s = m.ws - w * a.S;
+    m.qrow = ((size_t)(w * a.Hq + hkv * GQ + gq) * a.S + s);
+    return m;
+}
+
+// Query rotation of one fragment, split in two phases so that its few global loads can be issued BEFORE the
+// K/V tile loads (loads return in issue order, so a dependent wait would otherwise drain the whole KV
+// prefetch first) and consumed after them.  The kernel rotates over the full head dimension only (RotE == E,
+// what the models on this path use); other rotary widths are rotated by the standalone kernel first and
+// enter here as pre-rotated queries.  One work item = one 16-byte chunk pair (e, e + E/2) of one row; the
+// item count per thread is a compile-time constant.  Index convention of src/rope.cuh:18-51: both halves
+// read cos/sin at the first-half index.
+// PRE = the queries arrive already rotated, [F,W,Hq,S,E] (the hogwild_sdpa entry): one item = one chunk copy.
+template <class DT, int E, int ROWS, int QSTR, bool PRE>
+struct QueryRotation {
+    static constexpr int SZ = Elem<DT>::size;
+    static constexpr int CH = Chunk<DT>::CH;
+    static constexpr int IPR = PRE ? E / CH : E / (2 * CH);                  // items per row
+    static constexpr int NIT = (ROWS * IPR + NTHREADS - 1) / NTHREADS;       // items per thread
+
+    u32x4 xa[NIT];
+    u32x4 xb[PRE ? 1 : NIT];
+    f32x4 cs[PRE ? 1 : NIT][CH / 4], sn[PRE ? 1 : NIT][CH / 4];
+
+    __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid) {
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / IPR, slot = item % IPR;
+            // rows beyond R (MFMA padding) and threads beyond the item count read row 0: harmless, and keeps the
+            // loads out of divergent control flow
+            const int r = (item < ROWS * IPR && r0 + rr < a.R) ? r0 + rr : r0;
+            const RowMap rm = map_row(a, r, hkv, GQ);
+            const HW_GLOBAL char* qp = a.q + (rm.qrow * E + (PRE ? f * fstride : 0)) * SZ;
+            xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
+            if constexpr (!PRE) {
+                xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + IPR) * 16);
+                const size_t co = ((size_t)f * a.W * a.S + rm.ws) * E + slot * CH;
+#pragma unroll
+                for (int i = 0; i < CH / 4; ++i) {
+                    cs[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.cos + co + 4 * i);
+                    sn[it][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.sin + co + 4 * i);
+                }
+            }
+        }
+    }
+
+    __device__ __forceinline__ void finish(const DevHeader& a, char* q_lds, int f, int hkv, int r0, int GQ, bool write_rq,
+                                           int tid) const {
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / IPR, slot = item % IPR;
+            if (item >= ROWS * IPR) continue;
+            char* lrow = q_lds + rr * QSTR;
+            const bool pad = r0 + rr >= a.R;   // padding rows of the 16-row MFMA block hold zeros
+            const u32x4 z = {0, 0, 0, 0};
+            if constexpr (PRE) {
+                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : xa[it];
+            } else {
+                float x1[CH], x2[CH], y1[CH], y2[CH];
+                Chunk<DT>::unpack(xa[it], x1);
+                Chunk<DT>::unpack(xb[it], x2);
+#pragma unroll
+                for (int i = 0; i < CH; ++i) {
+                    const float c = cs[it][i >> 2][i & 3], sv = sn[it][i >> 2][i & 3];
+                    y1[i] = x1[i] * c - x2[i] * sv;
+                    y2[i] = x2[i] * c + x1[i] * sv;
+                }
+                const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
+                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : ya;
+                *reinterpret_cast<u32x4*>(lrow + (slot + IPR) * 16) = pad ? z : yb;
+                if (write_rq && !pad) {
+                    const RowMap rm = map_row(a, r0 + rr, hkv, GQ);
+                    HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
+                    *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
+                    *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + IPR) * 16) = yb;
+                }
+            }
+        }
+    }
+};
+
+}  // namespace hw

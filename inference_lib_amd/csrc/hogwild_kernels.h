@@ -62,4 +62,47 @@ hipError_t launch_rope(void* out, const void* q, const float* cosv, const float*
 hipError_t launch_stream_read(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
 hipError_t launch_stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 
+// ---- paged variants: KV of worker w lives in blocks of a shared cache, found through a block table ----
+
+// Scalar arguments of the paged attention kernel: 48 dwords, fetched with three 64-byte scalar loads.
+// The queries, locations and the output use the layout [LW, Hq, LS]: (W, S) for the fixed-length operator,
+// (total_q, 1) for the packed variable-length one.
+struct alignas(64) PagedHeader {
+    const void* q;             // [F, LW, Hq, LS, E] rotated queries
+    const int* loc;            // [F, LW*LS]
+    const int* frag_len;       // [F] or, with cu_q, [F, W]
+    const void* kcache;        // [num_blocks, Hkv, block_size, E]
+    const void* vcache;        // [num_blocks, Hkv, block_size, Ev]
+    const int* block_table;    // [W, max_blocks]
+    const int* cu_q;           // [W + 1] query-token prefix sums, or null: worker w owns tokens w*LS .. (w+1)*LS-1
+    float* part_o;             // [Hkv][nsplit][R][Ev]
+    float* part_ml;            // [Hkv][nsplit][R][2]
+    int F, W, Hq, Hkv, LW, LS;
+    int R;                     // LW*LS*(Hq/Hkv): query rows per kv head
+    int block_size, max_blocks, num_blocks;
+    int nsplit;                // workgroups that share one (kv head, row group)
+    int nitems;                // row groups over all workers (an upper bound when cu_q is given)
+    int nrg;                   // row groups per worker (fixed-length operator)
+    int nwg;
+    int xcd_remap;
+    float sc;                  // scale * log2(e)
+    unsigned magic_gq, magic_ls, magic_bs, magic_nsplit, magic_nitems, magic_nrg;   // ceil(2^32 / d)
+    int pad[8];
+};
+static_assert(sizeof(PagedHeader) == 192, "PagedHeader must be 48 dwords");
+
+struct CopyBlocksArgs {
+    const void* key_states;    // [B, Hkv, S_new, E]   (element strides below, innermost contiguous)
+    const void* value_states;  // [B, Hkv, S_new, Ev]
+    void* kcache;
+    void* vcache;
+    const int* block_table;    // [B, max_blocks]
+    const int* seq_lengths;    // [B]
+    long long ks_b, ks_h, ks_s, vs_b, vs_h, vs_s;
+    int B, Hkv, S_new, E, Ev, block_size, max_blocks, num_blocks;
+};
+
+hipError_t launch_paged_attention(const PagedHeader& ph, int dtype, int E, int rb, hipStream_t stream);
+hipError_t launch_copy_to_blocks(const CopyBlocksArgs& ca, int dtype, hipStream_t stream);
+
 }  // namespace hw

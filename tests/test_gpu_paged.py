@@ -1,0 +1,249 @@
+"""GPU parity of the paged operators (hw_paged_sdpa, hw_varlen_paged_sdpa, hw_copy_to_blocks) against
+oracle/paged_oracle.py, through the C ABI.  Tolerances: bf16/fp16 2e-2, fp32 1e-4 (max abs, out and lse);
+copy_to_blocks is bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np64
+
+pytestmark = pytest.mark.gpu
+
+TDT = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def build_paged(dtype, F, W, Hq, Hkv, D, bs, max_blocks, seq_lens, S=None, q_lens=None, seed=0, poison=True,
+                frag_lens=None, loc_mode="causal"):
+    """Synthetic paged problem on the CPU.  seq_lens[w] = tokens in sequence w.  Either S (fixed-length operator) or
+    q_lens[w] (variable-length operator).  Blocks a sequence does not need are left NaN and their table entries hold
+    garbage, so any read outside the visible part of a sequence shows up in the result."""
+    g = torch.Generator().manual_seed(seed)
+    tdt = TDT[dtype]
+    NB = W * max_blocks + 5
+    kc = torch.full((NB, Hkv, bs, D), float("nan") if poison else 0.0, dtype=torch.float32)
+    vc = torch.full((NB, Hkv, bs, D), float("nan") if poison else 0.0, dtype=torch.float32)
+    perm = torch.randperm(NB, generator=g)[: W * max_blocks].reshape(W, max_blocks).to(torch.int32)
+    bt = perm.clone()
+    for w in range(W):
+        need = (seq_lens[w] + bs - 1) // bs
+        for b in range(need):
+            n_tok = min(bs, seq_lens[w] - b * bs)
+            kc[perm[w, b], :, :n_tok] = torch.randn((Hkv, n_tok, D), generator=g)
+            vc[perm[w, b], :, :n_tok] = torch.randn((Hkv, n_tok, D), generator=g)
+        bt[w, need:] = torch.tensor([-7, 2 ** 30, NB, -1] * max_blocks, dtype=torch.int32)[: max_blocks - need]
+    varlen = q_lens is not None
+    if varlen:
+        cu = torch.zeros(W + 1, dtype=torch.int32)
+        cu[1:] = torch.cumsum(torch.tensor(q_lens), 0)
+        T = int(cu[-1])
+        q = torch.randn((F, T, Hq, D), generator=g)
+        loc = torch.zeros((F, T), dtype=torch.int32)
+        fl = torch.zeros((F, W), dtype=torch.int32)
+        for w in range(W):
+            a, b = int(cu[w]), int(cu[w + 1])
+            for f in range(F):
+                fl[f, w] = seq_lens[w] if frag_lens is None else min(frag_lens[f], seq_lens[w])
+                if loc_mode == "causal":   # the last q_lens[w] positions of the sequence, shifted per fragment
+                    loc[f, a:b] = torch.arange(seq_lens[w] - (b - a), seq_lens[w], dtype=torch.int32) - 3 * f
+                else:
+                    loc[f, a:b] = torch.randint(-2, seq_lens[w] + 3, (b - a,), generator=g, dtype=torch.int32)
+    else:
+        cu = None
+        q = torch.randn((F, W, Hq, S, D), generator=g)
+        loc = torch.zeros((F, W, S), dtype=torch.int32)
+        # a fragment length applies to all workers: it may not exceed the shortest sequence (longer would be unwritten cache)
+        fl = torch.tensor([min(seq_lens) if frag_lens is None else min(frag_lens[f], min(seq_lens)) for f in range(F)], dtype=torch.int32)
+        if frag_lens is None and F == 1:
+            fl[0] = max(seq_lens)          # visibility is then bounded by the locations alone
+        for w in range(W):
+            for f in range(F):
+                if loc_mode == "causal":
+                    loc[f, w] = torch.arange(seq_lens[w] - S, seq_lens[w], dtype=torch.int32) - 3 * f
+                else:
+                    loc[f, w] = torch.randint(-2, seq_lens[w], (S,), generator=g, dtype=torch.int32)
+    q = q.to(tdt)
+    kc = kc.to(tdt)
+    vc = vc.to(tdt)
+    return dict(q=q, loc=loc, fl=fl, kc=kc, vc=vc, bt=bt, cu=cu, scale=1.0 / D ** 0.5, dtype=dtype, F=F, W=W, Hq=Hq,
+                Hkv=Hkv, D=D, S=S)
+
+
+def oracle_paged(c):
+    from oracle import paged_oracle as po
+    kc = np.nan_to_num(np64(c["kc"]), nan=1e30)      # poisoned rows are never visible; keep the oracle's einsum finite
+    vc = np.nan_to_num(np64(c["vc"]), nan=1e30)
+    bt = np.clip(c["bt"].numpy(), 0, kc.shape[0] - 1)
+    if c["cu"] is None:
+        return po.paged_sdpa(np64(c["q"]), c["loc"].numpy(), c["fl"].numpy(), kc, vc, bt, c["scale"])
+    return po.varlen_paged_sdpa(np64(c["q"]), c["loc"].numpy(), c["fl"].numpy(), kc, vc, bt, c["cu"].numpy(), c["scale"])
+
+
+def run_paged(c, splits=0, row_blocks=0, with_lse=True):
+    from inference_lib_amd import _lib
+    dev = torch.device("cuda:0")
+    d = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in c.items()}
+    if c["cu"] is None:
+        out = torch.full((c["W"], c["Hq"], c["S"], c["D"]), float("nan"), dtype=d["q"].dtype, device=dev)
+    else:
+        out = torch.full((d["q"].size(1), c["Hq"], c["D"]), float("nan"), dtype=d["q"].dtype, device=dev)
+    lse = torch.full(out.shape[:-1], float("nan"), dtype=torch.float32, device=dev) if with_lse else None
+    pr = _lib.PagedProblem(q=d["q"], locations=d["loc"], fragment_lengths=d["fl"], key_cache=d["kc"], value_cache=d["vc"],
+                           block_table=d["bt"], scale=c["scale"], out=out, cu_seqlens_q=d["cu"], lse=lse, splits=splits,
+                           row_blocks=row_blocks)
+    print(f"paged run: dtype={c['dtype']} F={c['F']} W={c['W']} Hq={c['Hq']} Hkv={c['Hkv']} D={c['D']} S={c['S']} "
+          f"bs={c['kc'].size(2)} mb={c['bt'].size(1)} varlen={c['cu'] is not None} splits={splits} rb={row_blocks}", flush=True)
+    pr.run()
+    torch.cuda.synchronize()
+    return out, lse
+
+
+def check(c, **kw):
+    want_o, want_l = oracle_paged(c)
+    out, lse = run_paged(c, **kw)
+    tol = TOL[c["dtype"]]
+    assert_close("out", out, want_o, tol)
+    assert_close("lse", lse, want_l, tol)
+    return out, lse
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("D", [128, 64])
+@pytest.mark.parametrize("bs,S,F", [(16, 1, 1), (32, 1, 1), (8, 3, 2), (1, 2, 1), (24, 1, 2), (128, 4, 1)])
+def test_paged_small(dtype, D, bs, S, F):
+    mb = max(1, 300 // bs)
+    c = build_paged(dtype, F, 3, 10, 2, D, bs, mb, seq_lens=[200, 37, 1 + S + 3 * F], S=S, seed=bs + S)
+    check(c)
+
+
+def test_paged_random_locations_and_fragment_lengths():
+    c = build_paged("bf16", 3, 4, 8, 2, 128, 16, 40, seq_lens=[600, 64, 333, 17], S=2, seed=5, frag_lens=[9, 17, 16], loc_mode="random")
+    check(c)
+
+
+@pytest.mark.parametrize("splits", [1, 3, 16])
+@pytest.mark.parametrize("row_blocks", [1, 2])
+def test_paged_split_and_row_block_invariance(splits, row_blocks):
+    c = build_paged("bf16", 1, 2, 8, 2, 128, 16, 80, seq_lens=[1000, 129], S=6, seed=11)
+    check(c, splits=splits, row_blocks=row_blocks)
+
+
+def test_paged_qwq_shape_decode():
+    """The headline model shape as a paged decode step: 4 workers with their own 3-4k-token sequences."""
+    c = build_paged("bf16", 1, 4, 40, 8, 128, 16, 256, seq_lens=[4096, 3001, 3500, 2048], S=1, seed=3)
+    out, lse = check(c)
+    out2, lse2 = run_paged(c)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)     # deterministic
+
+
+def test_paged_gqa16_and_wide_rows():
+    c = build_paged("f16", 1, 2, 32, 2, 128, 32, 20, seq_lens=[500, 77], S=5, seed=9)     # 80 rows per worker
+    check(c)
+
+
+def test_paged_nothing_visible():
+    c = build_paged("bf16", 1, 2, 4, 2, 64, 16, 4, seq_lens=[20, 20], S=1, seed=1)
+    c["loc"][:, 0] = -1
+    out, lse = check(c)
+    assert (out[0] == 0).all() and torch.isneginf(lse[0]).all()
+
+
+@pytest.mark.parametrize("dtype,D", [("bf16", 128), ("f32", 64), ("f16", 64)])
+def test_varlen_ragged(dtype, D):
+    c = build_paged(dtype, 2, 5, 10, 2, D, 16, 30, seq_lens=[400, 50, 9, 130, 64], q_lens=[3, 0, 9, 40, 1], seed=21)
+    check(c)
+
+
+def test_varlen_many_sequences():
+    W = 150     # more than one 64-wide chunk of the sequence lookup
+    rng = np.random.default_rng(4)
+    seq = [int(x) for x in rng.integers(5, 90, size=W)]
+    ql = [int(min(s, x)) for s, x in zip(seq, rng.integers(0, 4, size=W))]
+    c = build_paged("bf16", 1, W, 4, 2, 64, 16, 6, seq_lens=seq, q_lens=ql, seed=8, loc_mode="random")
+    check(c)
+
+
+def test_varlen_equals_fixed_when_lengths_are_equal():
+    c = build_paged("bf16", 1, 3, 8, 2, 128, 16, 20, seq_lens=[300, 200, 100], S=4, seed=2)
+    out, lse = run_paged(c)
+    v = dict(c)
+    v["q"] = c["q"].permute(0, 1, 3, 2, 4).reshape(1, 12, 8, 128).contiguous()
+    v["loc"] = c["loc"].reshape(1, 12).contiguous()
+    v["fl"] = c["fl"][:, None].repeat(1, 3).contiguous()
+    v["cu"] = torch.arange(4, dtype=torch.int32) * 4
+    vo, vl = run_paged(v)
+    assert torch.equal(vo, out.permute(0, 2, 1, 3).reshape(12, 8, 128))
+    assert torch.equal(vl, lse.permute(0, 2, 1).reshape(12, 8))
+
+
+# --------------------------------------------------------------------------------------------------- copy_to_blocks
+@pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
+@pytest.mark.parametrize("E,Ev,S_new,bs", [(128, 128, 1, 16), (64, 64, 37, 16), (128, 64, 5, 1), (6, 10, 3, 4), (128, 128, 9, 24)])
+def test_copy_to_blocks_bit_exact(dtype, E, Ev, S_new, bs):
+    from inference_lib_amd import _lib
+    from oracle import paged_oracle as po
+    g = torch.Generator().manual_seed(S_new + bs)
+    tdt = TDT[dtype]
+    B, Hkv, mb = 3, 2, (60 + S_new) // bs + 2
+    NB = B * mb + 2
+    kc = torch.randn((NB, Hkv, bs, E), generator=g).to(tdt)
+    vc = torch.randn((NB, Hkv, bs, Ev), generator=g).to(tdt)
+    bt = torch.randperm(NB, generator=g)[: B * mb].reshape(B, mb).to(torch.int32)
+    seq = torch.tensor([0, 17, 60], dtype=torch.int32)
+    # the usual layout of fresh projections: [B, S_new, Hkv, D], viewed as [B, Hkv, S_new, D]
+    ks = torch.randn((B, S_new, Hkv, E), generator=g).to(tdt).transpose(1, 2)
+    vs = torch.randn((B, S_new, Hkv, Ev), generator=g).to(tdt).transpose(1, 2)
+    want_k, want_v = np64(kc), np64(vc)
+    po.copy_to_blocks(np64(ks), np64(vs), want_k, want_v, bt.numpy(), seq.numpy())
+    dev = torch.device("cuda:0")
+    dk, dv = kc.to(dev), vc.to(dev)
+    print(f"copy_to_blocks: {dtype} E={E} Ev={Ev} S_new={S_new} bs={bs}", flush=True)
+    _lib.copy_to_blocks(ks.to(dev), vs.to(dev), dk, dv, bt.to(dev), seq.to(dev))
+    torch.cuda.synchronize()
+    assert np.array_equal(np64(dk), want_k) and np.array_equal(np64(dv), want_v)
+
+
+def test_copy_to_blocks_skips_positions_outside_the_table():
+    from inference_lib_amd import _lib
+    dev = torch.device("cuda:0")
+    kc = torch.zeros((4, 1, 4, 8), dtype=torch.float16, device=dev)
+    vc = torch.zeros((4, 1, 4, 8), dtype=torch.float16, device=dev)
+    bt = torch.tensor([[2, 9]], dtype=torch.int32, device=dev)        # second entry lies outside the cache
+    seq = torch.tensor([2], dtype=torch.int32, device=dev)
+    ks = torch.ones((1, 1, 9, 8), dtype=torch.float16, device=dev)    # positions 2..10: 2,3 land; 4..7 bad block; 8.. off the table
+    _lib.copy_to_blocks(ks, ks, kc, vc, bt, seq)
+    torch.cuda.synchronize()
+    assert float(kc.sum()) == 2 * 8 and float(kc[2, 0, 2:].sum()) == 16 and float(vc.sum()) == 16
+
+
+def test_append_then_attend_round_trip():
+    """Decode loop in miniature: append one token per sequence with copy_to_blocks, then attend over the grown cache."""
+    from inference_lib_amd import _lib
+    from oracle import paged_oracle as po
+    dev = torch.device("cuda:0")
+    c = build_paged("bf16", 1, 3, 8, 2, 128, 16, 10, seq_lens=[100, 31, 64], S=1, seed=13, poison=False)
+    g = torch.Generator().manual_seed(99)
+    ks = torch.randn((3, 2, 1, 128), generator=g).to(torch.bfloat16)
+    vs = torch.randn((3, 2, 1, 128), generator=g).to(torch.bfloat16)
+    seq = torch.tensor([100, 31, 64], dtype=torch.int32)
+    bt = c["bt"].clone()
+    # give every sequence a valid block for its position seq_len (the builder left garbage beyond the used blocks)
+    used = set(int(x) for w in range(3) for x in bt[w, : (seq[w] + 15) // 16])
+    free = [b for b in range(c["kc"].size(0)) if b not in used]
+    for w in range(3):
+        if int(seq[w]) % 16 == 0:
+            bt[w, int(seq[w]) // 16] = free.pop()
+    c["bt"] = bt
+    want_k, want_v = np64(c["kc"]), np64(c["vc"])
+    po.copy_to_blocks(np64(ks), np64(vs), want_k, want_v, bt.numpy(), seq.numpy())
+    c["loc"] = seq.reshape(1, 3, 1).clone()
+    c["fl"] = torch.tensor([200], dtype=torch.int32)
+    want_o, want_l = po.paged_sdpa(np64(c["q"]), c["loc"].numpy(), c["fl"].numpy(), want_k, want_v, bt.numpy(), c["scale"])
+    d = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in c.items()}
+    _lib.copy_to_blocks(ks.to(dev), vs.to(dev), d["kc"], d["vc"], d["bt"], seq.to(dev))
+    out = torch.empty((3, 8, 1, 128), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((3, 8, 1), dtype=torch.float32, device=dev)
+    _lib.PagedProblem(q=d["q"], locations=d["loc"], fragment_lengths=d["fl"], key_cache=d["kc"], value_cache=d["vc"],
+                      block_table=d["bt"], scale=c["scale"], out=out, lse=lse).run()
+    torch.cuda.synchronize()
+    assert_close("out", out, want_o, 2e-2)
+    assert_close("lse", lse, want_l, 2e-2)
