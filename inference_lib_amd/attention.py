@@ -77,3 +77,51 @@ def hogwild_rope(queries: torch.Tensor, cosines: torch.Tensor, sines: torch.Tens
         torch.ops.libhogatt.hogwild_rope(out, queries, cosines, sines)
         return out
     return _lib.rope(queries, cosines, sines, out)
+
+
+def hogwild_paged_sdpa(queries: torch.Tensor, locations: torch.Tensor, fragment_lengths: torch.Tensor, key_cache: torch.Tensor,
+                       value_cache: torch.Tensor, block_table: torch.Tensor, scale: float, out=None,
+                       lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of rotated queries [F,W,Hq,S,E] over paged sequences (operator `hogwild_paged_sdpa`,
+    src/binding.cu:269-281; the reference has no Python wrapper for it).  `lse` (float32 [W,Hq,S]) is an addition and
+    goes through the C ABI directly."""
+    if out is None:
+        out = torch.empty((queries.size(1), queries.size(2), queries.size(3), value_cache.size(-1)), dtype=queries.dtype,
+                          device=queries.device)
+    if HAVE_TORCH_OPS and lse is None:
+        torch.ops.libhogatt.hogwild_paged_sdpa(out, scale, locations, queries.contiguous(), fragment_lengths, key_cache,
+                                               value_cache, block_table)
+        return out
+    _lib.PagedProblem(q=queries.contiguous(), locations=locations, fragment_lengths=fragment_lengths, key_cache=key_cache,
+                      value_cache=value_cache, block_table=block_table, scale=scale, out=out, lse=lse).run()
+    return out
+
+
+def hogwild_varlen_paged_sdpa(queries: torch.Tensor, locations: torch.Tensor, fragment_lengths: torch.Tensor,
+                              key_cache: torch.Tensor, value_cache: torch.Tensor, block_table: torch.Tensor,
+                              cu_seqlens_q: torch.Tensor, cu_seqlens_k: Optional[torch.Tensor], scale: float, out=None,
+                              lse: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Packed variable-length form: queries [F,total_q,Hq,E], locations [F,total_q], fragment_lengths [F,W]
+    (operator `hogwild_varlen_paged_sdpa`, src/binding.cu:283-296).  `cu_seqlens_k` is accepted and unused, as in the
+    reference's kernel."""
+    if out is None:
+        out = torch.empty((queries.size(1), queries.size(2), value_cache.size(-1)), dtype=queries.dtype, device=queries.device)
+    if HAVE_TORCH_OPS and lse is None:
+        torch.ops.libhogatt.hogwild_varlen_paged_sdpa(out, scale, locations, queries.contiguous(), fragment_lengths, key_cache,
+                                                      value_cache, block_table, cu_seqlens_q,
+                                                      cu_seqlens_k if cu_seqlens_k is not None else cu_seqlens_q)
+        return out
+    _lib.PagedProblem(q=queries.contiguous(), locations=locations, fragment_lengths=fragment_lengths, key_cache=key_cache,
+                      value_cache=value_cache, block_table=block_table, scale=scale, out=out, cu_seqlens_q=cu_seqlens_q,
+                      lse=lse).run()
+    return out
+
+
+def copy_to_blocks(key_states: torch.Tensor, value_states: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor,
+                   block_table: torch.Tensor, seq_lengths: torch.Tensor) -> None:
+    """Append new K/V rows [B,Hkv,S_new,D] to the paged caches at positions seq_lengths[b] + t (operator
+    `copy_to_blocks`, src/binding.cu:310-322)."""
+    if HAVE_TORCH_OPS:
+        torch.ops.libhogatt.copy_to_blocks(key_states, value_states, key_cache, value_cache, block_table, seq_lengths)
+        return
+    _lib.copy_to_blocks(key_states, value_states, key_cache, value_cache, block_table, seq_lengths)

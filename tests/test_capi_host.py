@@ -156,3 +156,97 @@ def test_no_fallback_when_library_is_missing(tmp_path, monkeypatch):
     r = subprocess.run([sys.executable, "-c", "import inference_lib_amd.attention"], cwd=tmp_path, capture_output=True, text=True,
                        env={**os.environ, "PYTHONPATH": str(tmp_path)})
     assert r.returncode != 0 and "libhogwild_hip.so" in r.stderr
+
+
+# ------------------------------------------------------------------------------------------------ paged entry points
+def test_paged_struct_layouts_match_header():
+    import shutil
+    import subprocess
+    import tempfile
+    L = _lib()
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "s.c")
+        open(src, "w").write('#include <stdio.h>\n#include <stddef.h>\n#include "hogwild_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu %zu %zu\\n",'
+                             'sizeof(hw_paged_problem),sizeof(hw_paged_plan),sizeof(hw_copy_blocks),offsetof(hw_paged_problem,cu_seqlens_q),'
+                             'offsetof(hw_paged_problem,row_blocks),offsetof(hw_copy_blocks,vs_s),offsetof(hw_copy_blocks,seq_lengths));return 0;}\n')
+        exe = os.path.join(d, "s")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)
+        out = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
+    assert out == [C.sizeof(L.HwPagedProblem), C.sizeof(L.HwPagedPlan), C.sizeof(L.HwCopyBlocks), L.HwPagedProblem.cu_seqlens_q.offset,
+                   L.HwPagedProblem.row_blocks.offset, L.HwCopyBlocks.vs_s.offset, L.HwCopyBlocks.seq_lengths.offset]
+
+
+def _paged(L, **over):
+    p = L.HwPagedProblem()
+    p.dtype, p.F, p.W, p.Hq, p.Hkv, p.E, p.Ev, p.S = L.HW_BF16, 1, 4, 40, 8, 128, 128, 1
+    p.block_size, p.max_blocks, p.num_blocks = 16, 256, 2000
+    p.scale = 0.1
+    for f in ("out", "q", "locations", "fragment_lengths", "key_cache", "value_cache", "block_table"):
+        setattr(p, f, 0x1000)                       # never dereferenced on the host
+    for key, val in over.items():
+        setattr(p, key, val)
+    return p
+
+
+def test_paged_validation_happens_on_the_host():
+    L = _lib()
+    v = lambda p: L.lib.hw_paged_validate(C.byref(p))
+    assert v(_paged(L)) == 0
+    assert L.lib.hw_paged_validate(None) == -1
+    assert v(_paged(L, dtype=5)) == -2
+    assert v(_paged(L, F=0)) == -5 and v(_paged(L, F=33)) == -5
+    assert v(_paged(L, Hq=41)) == -3
+    assert v(_paged(L, scale=0.0)) == -3 and v(_paged(L, scale=float("nan"))) == -3
+    assert v(_paged(L, block_size=0)) == -3 and v(_paged(L, block_size=4096)) == -3
+    assert v(_paged(L, max_blocks=70000)) == -3                      # more than 2^20 positions per sequence
+    assert v(_paged(L, num_blocks=1 << 25)) == -3                    # 2^31 cache rows
+    assert v(_paged(L, key_cache=None)) == -1
+    assert v(_paged(L, q=0x1008)) == -7
+    assert v(_paged(L, E=96, Ev=96)) == -4
+    assert v(_paged(L, S=0)) == -3
+    assert v(_paged(L, S=0, total_q=77, cu_seqlens_q=0x1000)) == 0   # the variable-length operator ignores S
+    # entry points reject the wrong operator before any device work
+    assert L.lib.hw_paged_sdpa(C.byref(_paged(L, cu_seqlens_q=0x1000)), None) == -3
+    assert L.lib.hw_varlen_paged_sdpa(C.byref(_paged(L)), None) == -1
+    assert L.lib.hw_paged_sdpa_stages(C.byref(_paged(L)), None, 0) == -3
+
+
+def test_paged_plan_invariants():
+    L = _lib()
+    # plain decode at the headline model shape: one 16-row block per worker and kv head, the CUs filled once
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1)
+    assert (pl.rows, pl.row_blocks, pl.row_groups) == (20, 1, 4)
+    assert pl.workgroups == 8 * 4 * pl.splits and pl.workgroups <= 256 and pl.splits >= 1
+    assert pl.workspace_bytes >= 8 * pl.splits * 20 * 130 * 4
+    # short sequences: never more waves than tiles at the longest sequence the table allows
+    pl = L.paged_plan(W=1, Hq=8, Hkv=8, Ev=128, block_size=16, max_blocks=8, num_cus=256, S=1)
+    assert pl.splits == 1
+    # many query tokens per worker: two row blocks, several row groups
+    pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20)
+    assert pl.row_blocks == 2 and pl.row_groups == 2 * 4
+    # fp32 exists with one row block only
+    pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20, dtype=L.HW_F32)
+    assert pl.row_blocks == 1 and pl.row_groups == 2 * 7
+    # variable length: the row-group count is an upper bound over every way of cutting total_q into W sequences
+    pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700)
+    assert pl.rows == 3500 and pl.row_groups >= 8 + 3500 // 32 and pl.workgroups == 8 * pl.row_groups * pl.splits
+    # explicit split factor is honoured (capped at 64)
+    assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=5).splits == 5
+    assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=500).splits == 64
+
+
+def test_copy_to_blocks_validation():
+    L = _lib()
+    c = L.HwCopyBlocks()
+    c.dtype, c.B, c.Hkv, c.S_new, c.E, c.Ev = L.HW_BF16, 2, 2, 1, 128, 128
+    c.block_size, c.max_blocks, c.num_blocks = 16, 4, 10
+    assert L.lib.hw_copy_to_blocks(None, None) == -1
+    assert L.lib.hw_copy_to_blocks(C.byref(c), None) == -1           # pointers missing
+    c.dtype = 9
+    assert L.lib.hw_copy_to_blocks(C.byref(c), None) == -2
+    c.dtype, c.block_size = L.HW_BF16, 0
+    assert L.lib.hw_copy_to_blocks(C.byref(c), None) == -3
+    c.block_size, c.S_new = 16, 0
+    assert L.lib.hw_copy_to_blocks(C.byref(c), None) == 0            # nothing to append: success without a device

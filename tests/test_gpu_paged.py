@@ -247,3 +247,50 @@ def test_append_then_attend_round_trip():
     torch.cuda.synchronize()
     assert_close("out", out, want_o, 2e-2)
     assert_close("lse", lse, want_l, 2e-2)
+
+
+# --------------------------------------------------------------------------------------------------- torch operators
+def test_paged_torch_ops_match_c_abi_and_raise_loudly():
+    from inference_lib_amd import attention
+    assert attention.HAVE_TORCH_OPS, "hogatt.abi3.so not built"
+    for name in ("hogwild_paged_sdpa", "copy_to_blocks", "hogwild_varlen_paged_sdpa"):
+        assert hasattr(torch.ops.libhogatt, name)
+    dev = torch.device("cuda:0")
+    c = build_paged("bf16", 2, 3, 10, 2, 128, 16, 12, seq_lens=[150, 40, 99], S=2, seed=31)
+    want_o, _ = oracle_paged(c)
+    d = {k: (v.to(dev) if torch.is_tensor(v) else v) for k, v in c.items()}
+    out = attention.hogwild_paged_sdpa(d["q"], d["loc"], d["fl"], d["kc"], d["vc"], d["bt"], c["scale"])
+    torch.cuda.synchronize()
+    assert_close("paged op", out, want_o, 2e-2)
+    ref, _ = run_paged(c)
+    assert torch.equal(out, ref)
+
+    v = build_paged("f16", 1, 4, 8, 2, 64, 16, 12, seq_lens=[150, 40, 99, 12], q_lens=[5, 0, 2, 12], seed=32)
+    want_o, _ = oracle_paged(v)
+    dv = {k: (t.to(dev) if torch.is_tensor(t) else t) for k, t in v.items()}
+    out = attention.hogwild_varlen_paged_sdpa(dv["q"], dv["loc"], dv["fl"], dv["kc"], dv["vc"], dv["bt"], dv["cu"], None, v["scale"])
+    torch.cuda.synchronize()
+    assert_close("varlen op", out, want_o, 2e-2)
+
+    # copy_to_blocks through the operator, with the transposed view a projection produces
+    kc, vc = d["kc"].clone(), d["vc"].clone()
+    ks = torch.randn((3, 4, 2, 128), device=dev).to(torch.bfloat16).transpose(1, 2)
+    seq = torch.tensor([150, 40, 99], dtype=torch.int32, device=dev)
+    bt = d["bt"].clone()
+    bt[:, 9] = torch.tensor([0, 1, 2], dtype=torch.int32, device=dev)
+    attention.copy_to_blocks(ks, ks, kc, vc, bt, seq)
+    kc2, vc2 = d["kc"].clone(), d["vc"].clone()
+    from inference_lib_amd import _lib
+    _lib.copy_to_blocks(ks, ks, kc2, vc2, bt, seq)
+    torch.cuda.synchronize()
+    assert torch.equal(kc.view(torch.int16), kc2.view(torch.int16)) and torch.equal(vc.view(torch.int16), vc2.view(torch.int16))
+
+    # unsupported head dimension and mismatched dtypes are errors, never silent no-ops
+    bad_kc = torch.zeros((4, 2, 16, 96), dtype=torch.bfloat16, device=dev)
+    bad_q = torch.zeros((1, 1, 4, 1, 96), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(RuntimeError, match="no kernel instantiated"):
+        attention.hogwild_paged_sdpa(bad_q, torch.zeros((1, 1, 1), dtype=torch.int32, device=dev),
+                                     torch.ones(1, dtype=torch.int32, device=dev), bad_kc, bad_kc,
+                                     torch.zeros((1, 2), dtype=torch.int32, device=dev), 1.0)
+    with pytest.raises(RuntimeError, match="dtype"):
+        torch.ops.libhogatt.hogwild_paged_sdpa(out.new_zeros((3, 10, 2, 128)), 1.0, d["loc"], d["q"].float(), d["fl"], d["kc"], d["vc"], d["bt"])
