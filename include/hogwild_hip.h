@@ -22,6 +22,10 @@
  *   hw_copy_to_blocks ...... copy_to_blocks           src/binding.cu:183-215, :310-322 (schema :371-372);
  *                            kernel src/cache.cuh:6-49
  *   hw_paged_problem ....... struct Shape with its paged / varlen members, src/common.h:5-20
+ *   hw_build_inputs ........ the layer-0 branch of HogwildCache.update, python/hogwild/attention.py:164-196
+ *                            (locations :173-181, model.rotary_emb + float cast :191-193)
+ *   hw_rope_append ......... apply_rotary_pos_emb on the new keys + the per-worker cache update,
+ *                            python/hogwild/attention.py:84-90, :313-318, :148-158; and merge_caches, :251-257
  */
 #ifndef HOGWILD_HIP_H
 #define HOGWILD_HIP_H
@@ -33,7 +37,7 @@
 extern "C" {
 #endif
 
-#define HW_ABI_VERSION 1
+#define HW_ABI_VERSION 2
 #define HW_MAX_FRAGMENTS 32
 #define HW_MAX_SPLITS 256      /* workgroups per kv head */
 
@@ -66,6 +70,8 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   cosines, sines [F, W, S, RotE] fp32      hw_fused_attention only (src/rope.cuh:18-51 index convention)
  *   k, v       HOST arrays of F device pointers; fragment f is [Hkv, len[f], E] / [Hkv, len[f], Ev]
  *   len        HOST array of F lengths (the reference reads the same numbers from the tensor sizes, src/binding.cu:91)
+ *   cap        optional HOST array of F row capacities: kv head h of fragment f starts h * cap[f] rows into its
+ *              buffers (a segment that grows in place inside a [Hkv, cap, D] allocation).  NULL = packed, cap == len.
  *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
@@ -93,6 +99,7 @@ typedef struct hw_problem {
     int32_t row_blocks;
     void* ev_start;
     void* ev_stop;
+    const int32_t* cap;
 } hw_problem;
 
 /* How a problem is cut into workgroups; filled by hw_plan_debug (host only, no device needed). */
@@ -227,6 +234,60 @@ typedef struct hw_copy_blocks {
 } hw_copy_blocks;
 
 int hw_copy_to_blocks(const hw_copy_blocks* c, void* stream);
+
+/* ------------------------------------------------------------------------------------------------------------
+ * Caller-side steps of a decode step (the reference does them in Python, python/hogwild/attention.py:137-204,251-257).
+ */
+
+/*
+ * locations[f,w,s] = pos_end[f*W + w] - S + s and the query rotation tables of those positions:
+ * cos/sin[f,w,s,i] = cos/sin(float(location) * inv_freq[i mod RotE/2]) * attention_scaling, fp32 arithmetic, rounded to
+ * `round_dtype` (HW_F32 = no rounding; the model library hands out the tables in the model dtype and the reference
+ * widens them back to fp32, python/hogwild/attention.py:191-193) and stored as fp32.
+ *   pos_end    HOST array [F, W]: for fragment f and worker w, the sum of the lengths of f and of every fragment that
+ *              follows f in worker w's order, new tokens included (python/hogwild/attention.py:174-181)
+ *   inv_freq   device fp32 [RotE/2]
+ *   locations  device int32 [F, W, S]; cosines / sines device fp32 [F, W, S, RotE]
+ */
+int hw_build_inputs(int32_t* locations, float* cosines, float* sines, const int32_t* pos_end, const float* inv_freq,
+                    float attention_scaling, int round_dtype, int F, int W, int S, int RotE, void* stream);
+
+#define HW_ROPE_EAGER 0   /* every product and the sum rounded as an eager tensor expression rounds them: bit-identical to
+                             apply_rotary_pos_emb of the reference on the same dtypes */
+#define HW_ROPE_FUSED 1   /* fp32 fused multiply-add, one rounding at the end */
+
+/*
+ * Rotate new keys and append keys and values to each worker's segment, in place:
+ *   K_dst[w][h, len[w] + t, :] = rope(key_states[w, h, S - n_new[w] + t, :], cos/sin[w, S - n_new[w] + t, :])
+ *   V_dst[w][h, len[w] + t, :] = value_states[w, h, S - n_new[w] + t, :]            t = 0 .. n_new[w]-1
+ * (left masking, python/hogwild/attention.py:149-155).  rope = (x * cos) + (rotate_half(x) * sin) on the first RotE
+ * elements, every element reading cos/sin at its own index (python/hogwild/attention.py:77-90); RotE == 0 appends
+ * without rotating (keys that arrive rotated).  Device pointers unless stated otherwise.
+ *   key_states / value_states   [W, Hkv, S, E|Ev] with element strides for the first three dimensions
+ *   cosines / sines             [W, S, RotE] with element strides cs_w, cs_s, in fp32 (cs_dtype == HW_F32) or in `dtype`
+ *                               (cs_dtype == dtype); cs_s == 0 applies one row to every token (merge_caches,
+ *                               python/hogwild/attention.py:252-256)
+ *   k_dst / v_dst               HOST arrays of W device pointers to segment buffers [Hkv, cap[w], E|Ev]
+ *   dst_len / dst_cap / n_new   HOST arrays of W ints; len + n_new <= cap is checked on the host
+ */
+typedef struct hw_append {
+    int32_t dtype, cs_dtype, mode;
+    int32_t W, Hkv, S, E, Ev, RotE;
+    const void* key_states;
+    const void* value_states;
+    int64_t ks_w, ks_h, ks_s;
+    int64_t vs_w, vs_h, vs_s;
+    const void* cosines;
+    const void* sines;
+    int64_t cs_w, cs_s;
+    void* const* k_dst;
+    void* const* v_dst;
+    const int32_t* dst_len;
+    const int32_t* dst_cap;
+    const int32_t* n_new;
+} hw_append;
+
+int hw_rope_append(const hw_append* a, void* stream);
 
 /* Number of compute units of the current device (0 on failure). */
 int hw_device_cus(void);

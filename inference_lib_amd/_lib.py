@@ -26,7 +26,7 @@ EXPORTS = [
     "hw_event_create", "hw_event_destroy", "hw_event_record", "hw_event_synchronize", "hw_event_elapsed_ms",
     "hw_stream_read", "hw_stream_copy",
     "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
-    "hw_paged_sdpa_stages", "hw_copy_to_blocks",
+    "hw_paged_sdpa_stages", "hw_copy_to_blocks", "hw_build_inputs", "hw_rope_append",
 ]
 
 
@@ -42,6 +42,7 @@ class HwProblem(C.Structure):
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("splits", C.c_int32), ("row_blocks", C.c_int32),
         ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p),
+        ("cap", C.POINTER(C.c_int32)),
     ]
 
 
@@ -90,6 +91,23 @@ class HwCopyBlocks(C.Structure):
     ]
 
 
+class HwAppend(C.Structure):
+    _fields_ = [
+        ("dtype", C.c_int32), ("cs_dtype", C.c_int32), ("mode", C.c_int32),
+        ("W", C.c_int32), ("Hkv", C.c_int32), ("S", C.c_int32), ("E", C.c_int32), ("Ev", C.c_int32), ("RotE", C.c_int32),
+        ("key_states", C.c_void_p), ("value_states", C.c_void_p),
+        ("ks_w", C.c_int64), ("ks_h", C.c_int64), ("ks_s", C.c_int64),
+        ("vs_w", C.c_int64), ("vs_h", C.c_int64), ("vs_s", C.c_int64),
+        ("cosines", C.c_void_p), ("sines", C.c_void_p),
+        ("cs_w", C.c_int64), ("cs_s", C.c_int64),
+        ("k_dst", C.POINTER(C.c_void_p)), ("v_dst", C.POINTER(C.c_void_p)),
+        ("dst_len", C.POINTER(C.c_int32)), ("dst_cap", C.POINTER(C.c_int32)), ("n_new", C.POINTER(C.c_int32)),
+    ]
+
+
+HW_ROPE_EAGER, HW_ROPE_FUSED = 0, 1
+
+
 class HogwildError(RuntimeError):
     def __init__(self, status: int, where: str):
         self.status = status
@@ -127,6 +145,9 @@ def _load() -> C.CDLL:
     lib.hw_varlen_paged_sdpa.argtypes = [C.POINTER(HwPagedProblem), C.c_void_p]
     lib.hw_paged_sdpa_stages.argtypes = [C.POINTER(HwPagedProblem), C.c_void_p, C.c_int]
     lib.hw_copy_to_blocks.argtypes = [C.POINTER(HwCopyBlocks), C.c_void_p]
+    lib.hw_build_inputs.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_void_p, C.c_float, C.c_int,
+                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.hw_rope_append.argtypes = [C.POINTER(HwAppend), C.c_void_p]
     return lib
 
 
@@ -140,6 +161,22 @@ def status_string(status: int) -> str:
 def check(status: int, where: str) -> None:
     if status != 0:
         raise HogwildError(status, where)
+
+
+def fragment_capacity(k: torch.Tensor, v: torch.Tensor) -> Optional[int]:
+    """Row capacity of a fragment whose tensors [Hkv, L, D] are views into [Hkv, cap, D] allocations (rows contiguous,
+    kv heads `cap` rows apart), or None if the pair is not of that form.  Packed fragments give cap == L."""
+    Hkv, L, E = k.shape
+    Ev = v.size(2)
+    if L == 0:
+        return 0
+    if (E > 1 and k.stride(2) != 1) or (Ev > 1 and v.stride(2) != 1) or (L > 1 and (k.stride(1) != E or v.stride(1) != Ev)):
+        return None
+    if Hkv == 1:
+        return L
+    if k.stride(0) % E != 0 or v.stride(0) % Ev != 0 or k.stride(0) // E != v.stride(0) // Ev or k.stride(0) // E < L:
+        return None
+    return k.stride(0) // E
 
 
 def _frag3(t: torch.Tensor) -> torch.Tensor:
@@ -178,13 +215,21 @@ class Problem:
             raise ValueError(f"queries have shape {tuple(q.shape)}, expected {expect_q}")
         if tuple(locations.shape) != (F, W, S) or locations.dtype != torch.int32:
             raise ValueError("locations must be int32 [F, W, S]")
-        tensors = [out, q, locations] + keys + values
+        tensors = [out, q, locations]
+        caps = []
         for f in range(F):
             if keys[f].size(0) != Hkv or values[f].size(0) != Hkv or keys[f].size(1) != values[f].size(1) \
                     or keys[f].size(2) != E or values[f].size(2) != Ev:
                 raise ValueError(f"fragment {f} has inconsistent shape")
             if keys[f].dtype != out.dtype or values[f].dtype != out.dtype:
                 raise ValueError("KV fragments must have the dtype of the output")
+            cap = fragment_capacity(keys[f], values[f])
+            if cap is None:
+                raise ValueError(f"fragment {f}: rows must be contiguous and kv heads a whole number of rows apart "
+                                 "(the same number for keys and values)")
+            caps.append(cap)
+            if keys[f].device != out.device or values[f].device != out.device:
+                raise ValueError("all tensors must live on the output's device")
         if q.dtype != out.dtype:
             raise ValueError("queries must have the dtype of the output")
         rot = 0
@@ -210,8 +255,9 @@ class Problem:
                 raise ValueError("all tensors must be contiguous")
             if t.device != out.device:
                 raise ValueError("all tensors must live on the output's device")
-        self._keep = tensors
+        self._keep = tensors + keys + values
         self.device = out.device
+        self._cap = (C.c_int32 * F)(*caps)
         self._k = (C.c_void_p * F)(*[k.data_ptr() for k in keys])
         self._v = (C.c_void_p * F)(*[v.data_ptr() for v in values])
         self._len = (C.c_int32 * F)(*[k.size(1) for k in keys])
@@ -229,6 +275,7 @@ class Problem:
         p.k = C.cast(self._k, C.POINTER(C.c_void_p))
         p.v = C.cast(self._v, C.POINTER(C.c_void_p))
         p.len = C.cast(self._len, C.POINTER(C.c_int32))
+        p.cap = C.cast(self._cap, C.POINTER(C.c_int32))
         p.splits = int(splits)
         p.row_blocks = int(row_blocks)
         self.p = p
@@ -447,6 +494,92 @@ def copy_to_blocks(key_states: torch.Tensor, value_states: torch.Tensor, key_cac
     with torch.cuda.device(key_cache.device):
         stream = torch.cuda.current_stream(key_cache.device).cuda_stream
         check(lib.hw_copy_to_blocks(C.byref(c), C.c_void_p(stream)), "hw_copy_to_blocks")
+
+
+def build_inputs(pos_end: Sequence[Sequence[int]], S: int, inv_freq: Optional[torch.Tensor], *, attention_scaling: float = 1.0,
+                 table_dtype: Optional[torch.dtype] = None, device=None):
+    """locations int32 [F, W, S], cosines / sines float32 [F, W, S, RotE] of a decode step.  pos_end[f][w] = position one
+    past the newest token of worker w as seen through fragment f (host numbers).  table_dtype = dtype the tables are
+    rounded to before being stored as float32 (None / float32: no rounding)."""
+    F, W = len(pos_end), len(pos_end[0])
+    flat = [int(x) for row in pos_end for x in row]
+    if len(flat) != F * W:
+        raise ValueError("pos_end must be a full [F][W] table")
+    rot = 0 if inv_freq is None else 2 * inv_freq.numel()
+    if inv_freq is not None:
+        if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous():
+            raise ValueError("inv_freq must be contiguous float32 [RotE/2]")
+        device = inv_freq.device
+    if device is None:
+        raise ValueError("a device is needed when there is no inv_freq tensor")
+    device = torch.device(device)
+    loc = torch.empty((F, W, S), dtype=torch.int32, device=device)
+    cos = torch.empty((F, W, S, rot), dtype=torch.float32, device=device)
+    sin = torch.empty((F, W, S, rot), dtype=torch.float32, device=device)
+    arr = (C.c_int32 * (F * W))(*flat)
+    rd = HW_F32 if table_dtype is None else _DTYPE_CODE[table_dtype]
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        check(lib.hw_build_inputs(loc.data_ptr(), cos.data_ptr(), sin.data_ptr(), arr,
+                                  inv_freq.data_ptr() if inv_freq is not None else None, float(attention_scaling), rd,
+                                  F, W, S, rot, C.c_void_p(stream)), "hw_build_inputs")
+    return loc, cos, sin
+
+
+def rope_append(key_states: torch.Tensor, value_states: torch.Tensor, k_dst: Sequence[torch.Tensor], v_dst: Sequence[torch.Tensor],
+                dst_len: Sequence[int], *, cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
+                n_new: Optional[Sequence[int]] = None, mode: int = HW_ROPE_EAGER) -> None:
+    """Rotate key_states [W, Hkv, S, E] with cosines / sines [W, S, RotE] (or [W, 1, RotE]: one row for all tokens) and
+    append keys and value_states [W, Hkv, S, Ev] to the segment buffers k_dst[w] / v_dst[w] ([Hkv, cap, E|Ev], contiguous)
+    behind their first dst_len[w] rows.  Without cosines the keys are appended as they are.  n_new[w] < S appends only
+    the last n_new[w] tokens of worker w."""
+    if key_states.dim() != 4 or value_states.dim() != 4 or key_states.shape[:3] != value_states.shape[:3]:
+        raise ValueError("key_states / value_states must be [W, Hkv, S, E|Ev]")
+    W, Hkv, S, E = key_states.shape
+    Ev = value_states.size(3)
+    if key_states.dtype not in _DTYPE_CODE or value_states.dtype != key_states.dtype:
+        raise HogwildError(-2, "rope_append")
+    if (E > 1 and key_states.stride(3) != 1) or (Ev > 1 and value_states.stride(3) != 1):
+        key_states, value_states = key_states.contiguous(), value_states.contiguous()
+    if len(k_dst) != W or len(v_dst) != W or len(dst_len) != W:
+        raise ValueError("one destination segment and length per worker")
+    for kd, vd in zip(k_dst, v_dst):
+        if kd.dim() != 3 or vd.dim() != 3 or kd.size(0) != Hkv or vd.size(0) != Hkv or kd.size(2) != E or vd.size(2) != Ev \
+                or kd.size(1) != vd.size(1) or not kd.is_contiguous() or not vd.is_contiguous():
+            raise ValueError("segment buffers must be contiguous [Hkv, cap, E|Ev] with one capacity for keys and values")
+        if kd.dtype != key_states.dtype or vd.dtype != key_states.dtype or kd.device != key_states.device:
+            raise ValueError("segment buffers must have the dtype and device of the new states")
+    a = HwAppend()
+    a.dtype = _DTYPE_CODE[key_states.dtype]
+    a.mode = int(mode)
+    a.W, a.Hkv, a.S, a.E, a.Ev = W, Hkv, S, E, Ev
+    a.key_states, a.value_states = key_states.data_ptr(), value_states.data_ptr()
+    a.ks_w, a.ks_h, a.ks_s = key_states.stride(0), key_states.stride(1), key_states.stride(2)
+    a.vs_w, a.vs_h, a.vs_s = value_states.stride(0), value_states.stride(1), value_states.stride(2)
+    a.cs_dtype = HW_F32
+    keep = [key_states, value_states]
+    if cosines is not None:
+        if sines is None or cosines.shape != sines.shape or cosines.dim() != 3 or cosines.size(0) != W or cosines.size(1) not in (1, S):
+            raise ValueError("cosines / sines must be [W, S, RotE] or [W, 1, RotE]")
+        if cosines.dtype != sines.dtype or cosines.dtype not in (torch.float32, key_states.dtype):
+            raise ValueError("cosines / sines must be float32 or have the dtype of the keys")
+        cosines, sines = cosines.contiguous(), sines.contiguous()
+        a.RotE = cosines.size(2)
+        a.cs_dtype = _DTYPE_CODE[cosines.dtype]
+        a.cosines, a.sines = cosines.data_ptr(), sines.data_ptr()
+        a.cs_w = cosines.stride(0)
+        a.cs_s = 0 if cosines.size(1) == 1 else cosines.stride(1)
+        keep += [cosines, sines]
+    kp = (C.c_void_p * W)(*[t.data_ptr() for t in k_dst])
+    vp = (C.c_void_p * W)(*[t.data_ptr() for t in v_dst])
+    ln = (C.c_int32 * W)(*[int(x) for x in dst_len])
+    cp = (C.c_int32 * W)(*[t.size(1) for t in k_dst])
+    nn = (C.c_int32 * W)(*([S] * W if n_new is None else [int(x) for x in n_new]))
+    a.k_dst, a.v_dst = C.cast(kp, C.POINTER(C.c_void_p)), C.cast(vp, C.POINTER(C.c_void_p))
+    a.dst_len, a.dst_cap, a.n_new = C.cast(ln, C.POINTER(C.c_int32)), C.cast(cp, C.POINTER(C.c_int32)), C.cast(nn, C.POINTER(C.c_int32))
+    with torch.cuda.device(key_states.device):
+        stream = torch.cuda.current_stream(key_states.device).cuda_stream
+        check(lib.hw_rope_append(C.byref(a), C.c_void_p(stream)), "hw_rope_append")
 
 
 def rope(q: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

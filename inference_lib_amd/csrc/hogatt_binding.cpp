@@ -51,11 +51,23 @@ at::Tensor fragment_view(const at::Tensor& t, const char* what, size_t f) {
     return t.dim() == 4 ? t.select(0, 0) : t;
 }
 
+// Rows between consecutive kv heads of a fragment [Hkv, L, D] whose rows are contiguous, or -1 if the pair of tensors is
+// not of that form (packed fragments give L).
+int64_t row_capacity(const at::Tensor& k, const at::Tensor& v) {
+    const int64_t Hkv = k.size(0), L = k.size(1), E = k.size(2), Ev = v.size(2);
+    if (L == 0) return 0;
+    if ((E > 1 && k.stride(2) != 1) || (Ev > 1 && v.stride(2) != 1)) return -1;
+    if (L > 1 && (k.stride(1) != E || v.stride(1) != Ev)) return -1;
+    if (Hkv == 1) return L;
+    if (k.stride(0) % E != 0 || v.stride(0) % Ev != 0 || k.stride(0) / E != v.stride(0) / Ev || k.stride(0) / E < L) return -1;
+    return k.stride(0) / E;
+}
+
 struct Unpacked {
     hw_problem p{};
     std::vector<at::Tensor> keep;          // contiguous fragment tensors kept alive until the launch is queued
     std::vector<const void*> kptr, vptr;
-    std::vector<int32_t> len;
+    std::vector<int32_t> len, cap;
     at::Tensor workspace;
 };
 
@@ -86,6 +98,7 @@ void unpack_common(Unpacked& u, at::Tensor& out, double scale, const at::Tensor&
     u.kptr.resize(F);
     u.vptr.resize(F);
     u.len.resize(F);
+    u.cap.resize(F);
     int64_t Hkv = -1;
     for (int64_t f = 0; f < F; ++f) {
         at::Tensor k = fragment_view(key_fragments[f], "key", f);
@@ -97,15 +110,21 @@ void unpack_common(Unpacked& u, at::Tensor& out, double scale, const at::Tensor&
         TORCH_CHECK(k.scalar_type() == out.scalar_type() && v.scalar_type() == out.scalar_type(),
                     "libhogatt: fragment ", f, " has a different dtype than the output");
         TORCH_CHECK(k.device() == out.device() && v.device() == out.device(), "libhogatt: fragment ", f, " lives on another device");
-        if (copy_noncontiguous) {   // the fused reference op does the same, src/binding.cu:330-337
+        // A fragment may be a view into a [Hkv, cap, D] allocation that grows in place: rows contiguous, kv heads a
+        // whole number of rows apart.  Anything else is copied by the fused op (as the reference does,
+        // src/binding.cu:330-337) and rejected by hogwild_sdpa.
+        int64_t cap = row_capacity(k, v);
+        if (cap < 0 && copy_noncontiguous) {
             k = k.contiguous();
             v = v.contiguous();
-        } else {
-            TORCH_CHECK(k.is_contiguous() && v.is_contiguous(), "libhogatt: fragment ", f, " must be contiguous");
+            cap = k.size(1);
         }
+        TORCH_CHECK(cap >= 0, "libhogatt: fragment ", f, " must be contiguous (or have contiguous rows and kv heads a whole "
+                    "number of rows apart, the same for keys and values)");
         u.kptr[f] = k.const_data_ptr();
         u.vptr[f] = v.const_data_ptr();
         u.len[f] = (int32_t)k.size(1);
+        u.cap[f] = (int32_t)cap;
         u.keep.push_back(k);
         u.keep.push_back(v);
     }
@@ -126,6 +145,7 @@ void unpack_common(Unpacked& u, at::Tensor& out, double scale, const at::Tensor&
     p.k = u.kptr.data();
     p.v = u.vptr.data();
     p.len = u.len.data();
+    p.cap = u.cap.data();
 }
 
 void run(Unpacked& u, const at::Tensor& out, bool fused) {

@@ -54,6 +54,7 @@ int validate(const hw_problem* p, int fused) {
     if ((long long)p->Hkv * ((rows + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
     for (int f = 0; f < p->F; ++f) {
         if (p->len[f] < 0) return HW_ERR_SHAPE;
+        if (p->cap != nullptr && p->cap[f] < p->len[f]) return HW_ERR_SHAPE;
         if (p->len[f] > 0 && (p->k[f] == nullptr || p->v[f] == nullptr)) return HW_ERR_NULL;
         if (!aligned16(p->k[f]) || !aligned16(p->v[f])) return HW_ERR_ALIGN;
         // one kv head of a fragment is addressed through a 32-bit buffer offset
@@ -187,6 +188,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
         ka.frag.k[f] = p->k[f];
         ka.frag.v[f] = p->v[f];
         ka.frag.len[f] = p->len[f];
+        ka.frag.cap[f] = p->cap != nullptr ? p->cap[f] : p->len[f];
     }
     for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
     for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];
@@ -391,6 +393,80 @@ int copy_blocks_run(const hw_copy_blocks* c, void* stream) {
     return (int)hw::launch_copy_to_blocks(a, c->dtype, reinterpret_cast<hipStream_t>(stream));
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// caller-side steps
+// ---------------------------------------------------------------------------------------------------------
+int build_inputs_run(int32_t* locations, float* cosines, float* sines, const int32_t* pos_end, const float* inv_freq,
+                     float scaling, int round_dtype, int F, int W, int S, int RotE, void* stream) {
+    if (F < 1 || W < 1 || S < 1 || RotE < 0 || (RotE & 1)) return HW_ERR_SHAPE;
+    if (round_dtype != HW_F32 && round_dtype != HW_F16 && round_dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (locations == nullptr || pos_end == nullptr) return HW_ERR_NULL;
+    if (RotE > 0 && (cosines == nullptr || sines == nullptr || inv_freq == nullptr)) return HW_ERR_NULL;
+    if (W > hw::MAX_POS_ENTRIES) return HW_ERR_UNSUPPORTED;
+    if ((long long)F * W * S * (RotE > 0 ? RotE : 1) >= (1ll << 31)) return HW_ERR_SHAPE;
+    const int fchunk = hw::MAX_POS_ENTRIES / W;      // fragments per launch
+    for (int f0 = 0; f0 < F; f0 += fchunk) {
+        const int nf = F - f0 < fchunk ? F - f0 : fchunk;
+        hw::BuildInputsArgs a;
+        a.locations = locations + (size_t)f0 * W * S;
+        a.cosines = RotE > 0 ? cosines + (size_t)f0 * W * S * RotE : nullptr;
+        a.sines = RotE > 0 ? sines + (size_t)f0 * W * S * RotE : nullptr;
+        a.inv_freq = inv_freq;
+        a.scaling = scaling;
+        a.F = nf; a.W = W; a.S = S; a.RotE = RotE;
+        std::memcpy(a.pos_end, pos_end + (size_t)f0 * W, sizeof(int) * (size_t)nf * W);
+        hipError_t e = hw::launch_build_inputs(a, round_dtype, reinterpret_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return (int)e;
+    }
+    return HW_OK;
+}
+
+int rope_append_run(const hw_append* p, void* stream) {
+    if (p == nullptr) return HW_ERR_NULL;
+    if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (p->cs_dtype != HW_F32 && p->cs_dtype != p->dtype) return HW_ERR_DTYPE;
+    if (p->mode != HW_ROPE_EAGER && p->mode != HW_ROPE_FUSED) return HW_ERR_SHAPE;
+    if (p->W < 1 || p->Hkv < 1 || p->S < 0 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
+    if (p->RotE < 0 || p->RotE > p->E || (p->RotE & 1)) return HW_ERR_SHAPE;
+    if (p->k_dst == nullptr || p->v_dst == nullptr || p->dst_len == nullptr || p->dst_cap == nullptr || p->n_new == nullptr) return HW_ERR_NULL;
+    bool any = false;
+    for (int w = 0; w < p->W; ++w) {
+        if (p->n_new[w] < 0 || p->n_new[w] > p->S || p->dst_len[w] < 0) return HW_ERR_SHAPE;
+        if ((long long)p->dst_len[w] + p->n_new[w] > p->dst_cap[w]) return HW_ERR_SHAPE;    // the segment is full
+        if (p->n_new[w] > 0) {
+            if (p->k_dst[w] == nullptr || p->v_dst[w] == nullptr) return HW_ERR_NULL;
+            any = true;
+        }
+    }
+    if (!any) return HW_OK;
+    if (p->key_states == nullptr || p->value_states == nullptr) return HW_ERR_NULL;
+    if (p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
+    for (int w0 = 0; w0 < p->W; w0 += hw::MAX_APPEND_WORKERS) {
+        const int nw = p->W - w0 < hw::MAX_APPEND_WORKERS ? p->W - w0 : hw::MAX_APPEND_WORKERS;
+        const size_t sz = elem_size(p->dtype), csz = p->cs_dtype == HW_F32 ? 4 : 2;
+        hw::AppendArgs a;
+        std::memset(&a, 0, sizeof(a));
+        a.k_src = reinterpret_cast<const char*>(p->key_states) + (long long)w0 * p->ks_w * (long long)sz;
+        a.v_src = reinterpret_cast<const char*>(p->value_states) + (long long)w0 * p->vs_w * (long long)sz;
+        a.cos = p->RotE > 0 ? reinterpret_cast<const char*>(p->cosines) + (long long)w0 * p->cs_w * (long long)csz : nullptr;
+        a.sin = p->RotE > 0 ? reinterpret_cast<const char*>(p->sines) + (long long)w0 * p->cs_w * (long long)csz : nullptr;
+        a.ks_w = p->ks_w; a.ks_h = p->ks_h; a.ks_s = p->ks_s;
+        a.vs_w = p->vs_w; a.vs_h = p->vs_h; a.vs_s = p->vs_s;
+        a.cs_w = p->cs_w; a.cs_s = p->cs_s;
+        a.W = nw; a.Hkv = p->Hkv; a.S = p->S; a.E = p->E; a.Ev = p->Ev; a.RotE = p->RotE;
+        for (int w = 0; w < nw; ++w) {
+            a.k_dst[w] = p->k_dst[w0 + w];
+            a.v_dst[w] = p->v_dst[w0 + w];
+            a.dst_len[w] = p->dst_len[w0 + w];
+            a.dst_cap[w] = p->dst_cap[w0 + w];
+            a.n_new[w] = p->n_new[w0 + w];
+        }
+        hipError_t e = hw::launch_rope_append(a, p->dtype, p->mode == HW_ROPE_EAGER, p->cs_dtype != HW_F32, reinterpret_cast<hipStream_t>(stream));
+        if (e != hipSuccess) return (int)e;
+    }
+    return HW_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -494,6 +570,13 @@ int hw_paged_sdpa_stages(const hw_paged_problem* p, void* stream, int stages) {
 }
 
 int hw_copy_to_blocks(const hw_copy_blocks* c, void* stream) { return copy_blocks_run(c, stream); }
+
+int hw_build_inputs(int32_t* locations, float* cosines, float* sines, const int32_t* pos_end, const float* inv_freq,
+                    float attention_scaling, int round_dtype, int F, int W, int S, int RotE, void* stream) {
+    return build_inputs_run(locations, cosines, sines, pos_end, inv_freq, attention_scaling, round_dtype, F, W, S, RotE, stream);
+}
+
+int hw_rope_append(const hw_append* a, void* stream) { return rope_append_run(a, stream); }
 
 int hw_device_cus(void) {
     int c = 0;

@@ -120,10 +120,10 @@ struct FragView {
 };
 constexpr unsigned OOB_OFFSET = 0xFFFF0000u;   // beyond any fragment (lengths are validated on the host)
 
-__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int krow, int vrow) {
+__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow) {
     FragView fv;
-    fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * L * krow), 0, L * krow, 0x00020000);
-    fv.v = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(vptr + (unsigned long long)hkv * L * vrow), 0, L * vrow, 0x00020000);
+    fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * cap * krow), 0, L * krow, 0x00020000);
+    fv.v = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(vptr + (unsigned long long)hkv * cap * vrow), 0, L * vrow, 0x00020000);
     return fv;
 }
 

@@ -18,6 +18,7 @@ struct FragTable {
     const void* k[MAXF];
     const void* v[MAXF];
     int len[MAXF];
+    int cap[MAXF];              // rows between consecutive kv heads of the fragment's buffers (>= len; == len when packed)
     int tile_begin[MAXF + 1];   // prefix sum of ceil(len/TILE): position of each fragment in a head's tile sequence
 };
 
@@ -104,5 +105,36 @@ struct CopyBlocksArgs {
 
 hipError_t launch_paged_attention(const PagedHeader& ph, int dtype, int E, int rb, hipStream_t stream);
 hipError_t launch_copy_to_blocks(const CopyBlocksArgs& ca, int dtype, hipStream_t stream);
+
+// ---- caller-side steps: input builder and fused key rotation + append ----
+constexpr int MAX_POS_ENTRIES = 768;    // (fragment, worker) pairs per build_inputs launch
+constexpr int MAX_APPEND_WORKERS = 64;  // workers per rope_append launch
+
+struct BuildInputsArgs {
+    int* locations;        // [F, W, S]
+    float* cosines;        // [F, W, S, RotE]
+    float* sines;
+    const float* inv_freq; // [RotE / 2]
+    float scaling;
+    int F, W, S, RotE;
+    int pos_end[MAX_POS_ENTRIES];   // [F][W]: position one past the newest token of worker w, as seen through fragment f
+};
+
+struct AppendArgs {
+    const void* k_src;     // [W, Hkv, S, E]  element strides ks_*, innermost contiguous
+    const void* v_src;     // [W, Hkv, S, Ev]
+    const void* cos;       // [W, S, RotE] element strides cs_w, cs_s (cs_s == 0 broadcasts one row over the tokens)
+    const void* sin;
+    long long ks_w, ks_h, ks_s, vs_w, vs_h, vs_s, cs_w, cs_s;
+    int W, Hkv, S, E, Ev, RotE;
+    void* k_dst[MAX_APPEND_WORKERS];     // segment buffers [Hkv, cap, E] / [Hkv, cap, Ev]
+    void* v_dst[MAX_APPEND_WORKERS];
+    int dst_len[MAX_APPEND_WORKERS];     // rows already in the segment
+    int dst_cap[MAX_APPEND_WORKERS];
+    int n_new[MAX_APPEND_WORKERS];       // the last n_new of the S source tokens are appended
+};
+
+hipError_t launch_build_inputs(const BuildInputsArgs& a, int round_dtype, hipStream_t stream);
+hipError_t launch_rope_append(const AppendArgs& a, int dtype, bool eager, bool cs16, hipStream_t stream);
 
 }  // namespace hw

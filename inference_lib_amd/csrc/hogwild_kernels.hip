@@ -94,6 +94,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
     const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
     const int my_len = args.frag.len[fl];
+    const int my_cap = args.frag.cap[fl];
     const int my_tb = args.frag.tile_begin[fl];
     const int my_te = args.frag.tile_begin[fl + 1];
     int my_wt[MAX_SPLITS / 64], my_wt1[MAX_SPLITS / 64];
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
                                       (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
         const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
                                       (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
-        const FragView fv = make_view(kp, vp, hkv, L, G::KROW, G::VROW);
+        const FragView fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW);
         const int lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
         const int lt1 = s1 - fb;
 

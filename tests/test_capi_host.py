@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
     for name in declared:
         assert hasattr(L.lib, name), name
-    assert L.lib.hw_version() == 1
+    assert L.lib.hw_version() == 2
 
 
 def test_struct_layout_matches_header():
@@ -250,3 +250,54 @@ def test_copy_to_blocks_validation():
     assert L.lib.hw_copy_to_blocks(C.byref(c), None) == -3
     c.block_size, c.S_new = 16, 0
     assert L.lib.hw_copy_to_blocks(C.byref(c), None) == 0            # nothing to append: success without a device
+
+
+# ------------------------------------------------------------------------------------------------ caller-side steps
+def test_append_struct_layout_matches_header():
+    import shutil
+    import subprocess
+    import tempfile
+    L = _lib()
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    with tempfile.TemporaryDirectory() as d:
+        src = os.path.join(d, "s.c")
+        open(src, "w").write('#include <stdio.h>\n#include <stddef.h>\n#include "hogwild_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu\\n",'
+                             'sizeof(hw_append),offsetof(hw_append,key_states),offsetof(hw_append,cs_s),offsetof(hw_append,n_new),'
+                             'offsetof(hw_problem,cap));return 0;}\n')
+        exe = os.path.join(d, "s")
+        subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)
+        out = [int(x) for x in subprocess.run([exe], check=True, capture_output=True, text=True).stdout.split()]
+    assert out == [C.sizeof(L.HwAppend), L.HwAppend.key_states.offset, L.HwAppend.cs_s.offset, L.HwAppend.n_new.offset,
+                   L.HwProblem.cap.offset]
+
+
+def test_build_inputs_and_append_validate_on_the_host():
+    L = _lib()
+    pe = (C.c_int32 * 4)(5, 6, 7, 8)
+    fake = 0x1000
+    bi = lambda **k: L.lib.hw_build_inputs(k.get("loc", fake), k.get("cos", fake), k.get("sin", fake), k.get("pe", pe), k.get("inv", fake),
+                                           1.0, k.get("rd", L.HW_F32), k.get("F", 2), k.get("W", 2), k.get("S", 1), k.get("R", 64), None)
+    assert bi(F=0) == -3 and bi(S=0) == -3 and bi(R=63) == -3 and bi(R=-2) == -3
+    assert bi(rd=9) == -2
+    assert bi(loc=None) == -1 and bi(pe=None) == -1 and bi(inv=None) == -1 and bi(cos=None) == -1
+    assert bi(W=769) == -4                                  # more workers than one launch can carry
+
+    def app(**k):
+        a = L.HwAppend()
+        a.dtype, a.cs_dtype, a.mode = k.get("dtype", L.HW_BF16), k.get("cs_dtype", L.HW_BF16), k.get("mode", 0)
+        a.W, a.Hkv, a.S, a.E, a.Ev, a.RotE = 1, 2, k.get("S", 4), 128, 128, k.get("RotE", 128)
+        a.key_states = a.value_states = a.cosines = a.sines = fake
+        kp = (C.c_void_p * 1)(k.get("dst", fake))
+        ln, cp, nn = (C.c_int32 * 1)(k.get("len", 3)), (C.c_int32 * 1)(k.get("cap", 16)), (C.c_int32 * 1)(k.get("n_new", 4))
+        a.k_dst = a.v_dst = C.cast(kp, C.POINTER(C.c_void_p))
+        a.dst_len, a.dst_cap, a.n_new = C.cast(ln, C.POINTER(C.c_int32)), C.cast(cp, C.POINTER(C.c_int32)), C.cast(nn, C.POINTER(C.c_int32))
+        a._keep = (kp, ln, cp, nn)
+        return L.lib.hw_rope_append(C.byref(a), None)
+    assert L.lib.hw_rope_append(None, None) == -1
+    assert app(dtype=5) == -2 and app(cs_dtype=L.HW_F16) == -2          # tables: float32 or the dtype of the keys
+    assert app(mode=2) == -3 and app(RotE=130) == -3 and app(RotE=7) == -3
+    assert app(n_new=5) == -3 and app(n_new=-1) == -3
+    assert app(len=13, n_new=4) == -3                                   # 13 + 4 rows do not fit a capacity of 16
+    assert app(dst=None) == -1
+    assert app(n_new=0) == 0                                            # nothing to append: success without a device
