@@ -185,6 +185,32 @@ def main():
         d2 = sorted(a.elapsed_ms(b) * 1e3 for a, b in evs2)
         kern_us_eager_med = d2[len(d2) // 2]
 
+        # ---------------- the caller-side steps of a decode step at this shape (latency-bound, tiny) ----------------
+        Hkv = cd.keys[0].size(0)
+        seg_k = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
+        seg_v = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
+        k_new = torch.randn((W, S, Hkv, E), device=dev).to(tdt).transpose(1, 2)
+        ck = torch.ones((W, S, E), dtype=tdt, device=dev)
+        inv = torch.ones(E // 2, dtype=torch.float32, device=dev)
+        pos_end = [[1000 + 7 * f + w for w in range(W)] for f in range(case.F)]
+        g_a = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_a, stream=stream):
+            for i in range(K):
+                _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck)
+        g_b = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_b, stream=stream):
+            for i in range(K):
+                _lib.build_inputs(pos_end, S, inv, table_dtype=tdt if tdt != torch.float32 else None)
+        side = []
+        for gr in (g_a, g_b):
+            gr.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            gr.replay()
+            torch.cuda.synchronize()
+            side.append((time.perf_counter() - t0) / K * 1e6)
+        append_us, build_us = side
+
         # ---------------- plain streaming read of the whole ring (achievable HBM rate) ----------------
         big = torch.empty(int(args.ring_mb * 1e6) // 16 * 16, dtype=torch.uint8, device=dev)
         big.random_(0, 255)
@@ -253,6 +279,8 @@ def main():
             "hot_cache_us_per_step": round(hot_us, 3),
             "hot_cache_GBps": round(kv_bytes / (hot_us * 1e-6) / 1e9, 1),
             "stream_read_GBps": round(stream_gbs, 1),
+            "rope_append_us_per_call": round(append_us, 3),
+            "build_inputs_us_per_call": round(build_us, 3),
             "timing": "K steps replayed as one HIP graph, wall clock between device synchronisations",
         },
     }

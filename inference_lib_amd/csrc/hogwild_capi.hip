@@ -187,8 +187,8 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     for (int f = 0; f < p->F; ++f) {
         ka.frag.k[f] = p->k[f];
         ka.frag.v[f] = p->v[f];
-        ka.frag.len[f] = p->len[f];
-        ka.frag.cap[f] = p->cap != nullptr ? p->cap[f] : p->len[f];
+        ka.frag.lc[f].len = p->len[f];
+        ka.frag.lc[f].cap = p->cap != nullptr ? p->cap[f] : p->len[f];
     }
     for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
     for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];

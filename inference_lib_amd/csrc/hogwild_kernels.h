@@ -17,8 +17,10 @@ constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary
 struct FragTable {
     const void* k[MAXF];
     const void* v[MAXF];
-    int len[MAXF];
-    int cap[MAXF];              // rows between consecutive kv heads of the fragment's buffers (>= len; == len when packed)
+    struct LenCap {
+        int len;                // tokens in the fragment
+        int cap;                // rows between consecutive kv heads of the fragment's buffers (>= len; == len when packed)
+    } lc[MAXF];                 // one 8-byte load per lane fetches both
     int tile_begin[MAXF + 1];   // prefix sum of ceil(len/TILE): position of each fragment in a head's tile sequence
 };
 

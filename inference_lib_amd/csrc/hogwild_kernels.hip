@@ -93,8 +93,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     const int fl = lane & (MAXF - 1);
     const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
     const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
-    const int my_len = args.frag.len[fl];
-    const int my_cap = args.frag.cap[fl];
+    const FragTable::LenCap my_lc = args.frag.lc[fl];
+    const int my_len = my_lc.len, my_cap = my_lc.cap;
     const int my_tb = args.frag.tile_begin[fl];
     const int my_te = args.frag.tile_begin[fl + 1];
     int my_wt[MAX_SPLITS / 64], my_wt1[MAX_SPLITS / 64];
