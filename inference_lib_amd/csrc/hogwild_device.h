@@ -10,6 +10,12 @@
 #ifndef HW_MARK
 #define HW_MARK(i) do { } while (0)
 #endif
+// Cache-policy bits of the K/V tile loads: 2 = non-temporal.  Every K/V byte is used exactly once per launch, so
+// the tiles are streamed past the caches instead of displacing the queries, tables and split-K partials
+// (measured: 17.35 -> 15.6 us per decode step at the 51 MB workload).
+#ifndef HW_KV_AUX
+#define HW_KV_AUX 2
+#endif
 
 namespace hw {
 
@@ -161,7 +167,7 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
     const unsigned kb = real ? (unsigned)(t0 * G::KROW) : OOB_OFFSET;
 #pragma unroll
     for (int i = 0; i < G::KL; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, HW_KV_AUX);
     // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load
     const unsigned vb = real ? (unsigned)((t0 + q * 4) * G::VROW + n * (G::VLD * 4)) : OOB_OFFSET;
 #pragma unroll
@@ -170,13 +176,13 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
 #pragma unroll
         for (int hh = 0; hh < G::NVL; ++hh) {
             if constexpr (G::VLD == 4) {
-                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(fv.v, vb + rowoff + hh * 256, 0, 0);
+                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(fv.v, vb + rowoff + hh * 256, 0, HW_KV_AUX);
                 t.v[idx][hh * 4 + 0] = x.x;
                 t.v[idx][hh * 4 + 1] = x.y;
                 t.v[idx][hh * 4 + 2] = x.z;
                 t.v[idx][hh * 4 + 3] = x.w;
             } else {
-                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(fv.v, vb + rowoff, 0, 0);
+                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(fv.v, vb + rowoff, 0, HW_KV_AUX);
                 t.v[idx][0] = x.x;
                 t.v[idx][1] = x.y;
             }

@@ -253,7 +253,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
             for (int i = 0; i < G::KL; ++i) {
                 const int r = __shfl(rid, i * RPL + lrow, 64);
                 const HW_GLOBAL char* src = ph.kcache + (unsigned long long)(unsigned)r * G::KROW + k_chunk(i);
-                __builtin_amdgcn_global_load_lds(src, HW_LDS_PTR(kslot + i * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(src, HW_LDS_PTR(kslot + i * 1024), 16, 0, HW_KV_AUX);
             }
 #pragma unroll
             for (int idx = 0; idx < 8; ++idx) {
@@ -262,13 +262,15 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
 #pragma unroll
                 for (int hh = 0; hh < G::NVL; ++hh) {
                     if constexpr (G::VLD == 4) {
-                        const u32x4 x = *reinterpret_cast<const HW_GLOBAL u32x4*>(src + hh * 256);
+                        const u32x4 x = HW_KV_AUX == 2 ? __builtin_nontemporal_load(reinterpret_cast<const HW_GLOBAL u32x4*>(src + hh * 256))
+                                                        : *reinterpret_cast<const HW_GLOBAL u32x4*>(src + hh * 256);
                         tr.v[idx][hh * 4 + 0] = x.x;
                         tr.v[idx][hh * 4 + 1] = x.y;
                         tr.v[idx][hh * 4 + 2] = x.z;
                         tr.v[idx][hh * 4 + 3] = x.w;
                     } else {
-                        const u32x2 x = *reinterpret_cast<const HW_GLOBAL u32x2*>(src);
+                        const u32x2 x = HW_KV_AUX == 2 ? __builtin_nontemporal_load(reinterpret_cast<const HW_GLOBAL u32x2*>(src))
+                                                        : *reinterpret_cast<const HW_GLOBAL u32x2*>(src);
                         tr.v[idx][0] = x.x;
                         tr.v[idx][1] = x.y;
                     }
