@@ -146,38 +146,50 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     HW_MARK(0);
     unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
 
-    while (todo != 0) {
-        const int f = __builtin_ctzll(todo);
+    // One segment = the part of a fragment that lies in this workgroup's tile range.  Opening a segment (decoding the
+    // tables, requesting its queries and its first tile) happens before the loop for the first one and at the bottom of
+    // the loop for the following ones, so that the requests of the first segment are on their way before the
+    // loop-invariant address arithmetic of the tile loop is computed.
+    int f = 0, L = 0, lt0 = 0, lt1 = 0;
+    bool opens_fragment = false;       // this workgroup owns the fragment's first tile (and writes its rotated queries)
+    FragView fv;
+    QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
+    int lm = 0;
+    TileRegs<DT, E, EV> tr[PF];
+    auto open_segment = [&]() {
+        f = __builtin_ctzll(todo);
         todo &= todo - 1;
         const int fb = __builtin_amdgcn_readlane(my_tb, f);
         const int fe = __builtin_amdgcn_readlane(my_te, f);
         const int s0 = max(T0, fb), s1 = min(T1, fe);
-        const int L = __builtin_amdgcn_readlane(my_len, f);
+        L = __builtin_amdgcn_readlane(my_len, f);
         const unsigned long long kp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_k >> 32), f) << 32) |
                                       (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
         const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
                                       (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
-        const FragView fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW);
-        const int lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
-        const int lt1 = s1 - fb;
-
-        // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first PF
-        // K/V tiles; the rotation then waits only for the former while the tiles stay in flight
+        fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW);
+        lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
+        lt1 = s1 - fb;
+        opens_fragment = s0 == fb;
+        // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first K/V tile; the
+        // rotation then waits only for the former while the tile stays in flight
         HW_MARK(6);
-        QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
         qrot.load(a, f, hkv, r0, GQ, tid);
         HW_MARK(7);
         // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
-        const int lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
+        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
         // the first tile is requested before the prologue, further look-ahead tiles after it: a wave stalls
         // while the memory pipeline accepts its requests, and the prologue should not sit behind that stall
-        TileRegs<DT, E, EV> tr[PF];
         if (PF > 1) load_tile<DT, E, EV>(tr[0], fv, kslots[0], koff, lt0 * TILE, n, q, lt0 < lt1);
+    };
+    bool more = todo != 0;
+    if (more) open_segment();
 
+    while (more) {
         HW_MARK(1);
         // ---- prologue: rotate the queries of this fragment into LDS ----
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
-        qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && s0 == fb, tid);
+        qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
         // rows that pad the MFMA block get "sees everything": their query is zero and they are never stored,
         // and they must not keep the unmasked fast path from being taken
         if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
@@ -230,6 +242,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
                 }
             }
         }
+        more = todo != 0;
+        if (more) open_segment();
     }
 
     HW_MARK(3);
@@ -242,12 +256,12 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     if (!PRE && a.rq != nullptr && g == 0) {
         unsigned long long empty = __ballot(lane < a.F && my_len == 0);
         while (empty != 0) {
-            const int f = __builtin_ctzll(empty);
+            f = __builtin_ctzll(empty);
             empty &= empty - 1;
             __syncthreads();
-            QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
-            qrot.load(a, f, hkv, r0, GQ, tid);
-            qrot.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
+            QueryRotation<DT, E, ROWS, G::QSTR, PRE> qempty;
+            qempty.load(a, f, hkv, r0, GQ, tid);
+            qempty.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
         }
     }
 }
