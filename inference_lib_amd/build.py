@@ -57,8 +57,21 @@ def build_torch_binding() -> str:
     return TORCH_EXT
 
 
+C_EXAMPLE = os.path.join(ROOT, "tests", "c_abi", "decode_step")
+
+
+def build_c_example() -> str:
+    """A caller of the C ABI in plain C (tests/c_abi/decode_step.c), linked against the library and the HIP runtime."""
+    cmd = ["gcc", "-std=c11", "-O1", "-Wall", "-D__HIP_PLATFORM_AMD__=1", "-I", os.path.join(ROOT, "include"), "-I", "/opt/rocm/include",
+           os.path.join(ROOT, "tests", "c_abi", "decode_step.c"), "-o", C_EXAMPLE, "-L", HERE, "-lhogwild_hip",
+           "-L", "/opt/rocm/lib", "-lamdhip64", "-lm", "-Wl,-rpath,$ORIGIN/../../inference_lib_amd", "-Wl,-rpath,/opt/rocm/lib"]
+    _run(cmd)
+    return C_EXAMPLE
+
+
 def build_all(with_torch: bool = True) -> None:
     build_library()
+    build_c_example()
     if with_torch:
         build_torch_binding()
 
