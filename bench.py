@@ -33,6 +33,8 @@ METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 worke
 # separate runs, each scaled by what the same counter reads for the 256 MiB copy kernel this script launches:
 # 0.5 for FETCH_SIZE, 1.0 for WRITE_SIZE): 51.78 MB fetched + 3.03 MB written.  Workloads not measured: None.
 MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_810_000}
+# the same for hw::paged_attention_kernel at the default paged workload (4 x 12528 tokens, blocks of 16): 205.69 MB + 0.67 MB
+MEASURED_PAGED_TRAFFIC_BYTES = {(12528, 16): 206_360_000}
 
 
 def parse_args():
@@ -388,7 +390,8 @@ def bench_paged(args, dev):
                                f"block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "hw::paged_attention_kernel",
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": MEASURED_PAGED_TRAFFIC_BYTES.get((L, bs)),
+                     "kernel": "hw::paged_attention_kernel",
                      "kernel_us_avg": round(kern_us, 3),
                      "timing": "two HIP events around a graph replay of K attention-kernel launches (merge stage off), divided by K"},
         "extra": {"us_per_step": round(graph_us, 3), "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2),
