@@ -1,0 +1,71 @@
+"""Seeded random sweep of shapes through the fused and the paged operator against the oracles: fragment lengths around
+the 32-token tile size, empty fragments, random worker orders, every dtype and head dimension, 1..9 workers, several
+query tokens, GQA group sizes 1..7, explicit split factors, segments inside larger allocations.  Tolerances as in the
+other parity tests (bf16/fp16 2e-2, fp32 1e-4)."""
+import numpy as np
+import pytest
+import torch
+
+from helpers import TOL, assert_close, np64, oracle_fused, run_fused
+from test_gpu_paged import build_paged, check as check_paged
+
+pytestmark = pytest.mark.gpu
+
+EDGE = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 256, 257, 1000, 1023, 1025]
+
+
+def random_case(seed):
+    from inference_lib_amd import cases
+    rng = np.random.default_rng(seed)
+    dtype = ["bf16", "f16", "f32"][seed % 3]
+    E = [128, 64][(seed // 3) % 2]
+    W = int(rng.integers(1, 10))
+    S = int(rng.choice([1, 1, 1, 2, 3]))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    GQ = int(rng.integers(1, 8))
+    F = int(rng.integers(1, 13))
+    lens = [int(rng.choice(EDGE)) if rng.random() < 0.7 else int(rng.integers(0, 3000)) for _ in range(F)]
+    if sum(lens) == 0:
+        lens[0] = 40
+    orders = [list(rng.permutation(F)) for _ in range(W)]
+    g = torch.Generator().manual_seed(seed)
+    c = cases.build_case(f"rand{seed}", dtype, W, S, Hkv * GQ, Hkv, E, 1e4, lens, [[int(x) for x in o] for o in orders], g)
+    return c, int(rng.choice([0, 0, 1, 3, 7, 40]))
+
+
+@pytest.mark.parametrize("seed", range(36))
+def test_fused_random_shapes(oracle, seed):
+    c, splits = random_case(seed)
+    print(f"seed {seed}: {c.dtype} E={c.E} W={c.W} S={c.S} Hq={c.Hq} Hkv={c.Hkv} lens={c.lens} splits={splits}", flush=True)
+    want_o, want_l, want_rq = oracle_fused(oracle, c)
+    out, lse, rq = run_fused(c.to(torch.device("cuda:0")), splits=splits)
+    tol = TOL[c.dtype]
+    assert_close("out", out, want_o, tol)
+    assert_close("lse", lse, want_l, tol)
+    assert_close("rq", rq, want_rq, 1e-5 if c.dtype == "f32" else 3.2e-2)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_paged_random_shapes(seed):
+    rng = np.random.default_rng(1000 + seed)
+    dtype = ["bf16", "f16", "f32"][seed % 3]
+    D = [128, 64][(seed // 3) % 2]
+    W = int(rng.integers(1, 7))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    GQ = int(rng.integers(1, 8))
+    bs = int(rng.choice([1, 4, 8, 16, 16, 32, 48, 64, 256]))
+    F = int(rng.integers(1, 4))
+    varlen = bool(rng.random() < 0.4)
+    S = int(rng.choice([1, 1, 2, 5]))
+    longest = int(rng.choice([40, 130, 700, 2100]))
+    seq = [int(rng.integers(S + 3 * F + 1, longest + S + 3 * F + 2)) for _ in range(W)]
+    mb = (max(seq) + bs - 1) // bs + int(rng.integers(0, 3))
+    kw = dict(seed=seed, loc_mode="random" if rng.random() < 0.5 else "causal")
+    if varlen:
+        ql = [int(min(s - 3 * F, x)) for s, x in zip(seq, rng.integers(0, 7, size=W))]
+        if sum(ql) == 0:
+            ql[0] = 1
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, D, bs, mb, seq_lens=seq, q_lens=ql, **kw)
+    else:
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, D, bs, mb, seq_lens=seq, S=S, **kw)
+    check_paged(c, splits=int(rng.choice([0, 0, 1, 5])))
