@@ -118,18 +118,24 @@ struct TileRegs {
 };
 
 #define HW_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define HW_GLOBAL __attribute__((address_space(1)))
 
-// A fragment's K and V slices of one kv head as buffer resources: out-of-range rows read as zero, so tiles
-// need no address clamping, and a tile that does not exist costs no memory traffic at all.
+// A fragment's K and V slices of one kv head.  K goes through a buffer resource: out-of-range rows read as zero, so
+// its global->LDS transfers need no address clamping and a tile that does not exist costs no memory traffic.  V is
+// read with plain global loads (measured: a tile's rows land ~15 % sooner than through buffer loads), with rows beyond
+// the fragment redirected to its last row.
 struct FragView {
-    __amdgpu_buffer_rsrc_t k, v;
+    __amdgpu_buffer_rsrc_t k;
+    unsigned long long vbase;   // start of the kv head's V rows
+    int L;
 };
 constexpr unsigned OOB_OFFSET = 0xFFFF0000u;   // beyond any fragment (lengths are validated on the host)
 
 __device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow) {
     FragView fv;
     fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * cap * krow), 0, L * krow, 0x00020000);
-    fv.v = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(vptr + (unsigned long long)hkv * cap * vrow), 0, L * vrow, 0x00020000);
+    fv.vbase = vptr + (unsigned long long)hkv * cap * vrow;
+    fv.L = L;
     return fv;
 }
 
@@ -158,8 +164,7 @@ __device__ __forceinline__ void k_lane_offsets(unsigned* koff, int lane) {
 
 // Issue the loads of one tile: K by direct global->LDS transfers into `kslot` (this wave's part of a staging
 // slot), V into registers.  The number of load instructions is the same whether or not the tile exists, which
-// keeps the hardware wait counts exact on every path; a tile that does not exist reads out of range (zeros,
-// no memory traffic).
+// keeps the hardware wait counts exact on every path; a tile that does not exist costs (almost) no memory traffic.
 template <class DT, int E, int EV>
 __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView& fv, char* kslot, const unsigned* koff, int t0,
                                           int n, int q, bool real) {
@@ -168,21 +173,23 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
 #pragma unroll
     for (int i = 0; i < G::KL; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, HW_KV_AUX);
-    // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load
-    const unsigned vb = real ? (unsigned)((t0 + q * 4) * G::VROW + n * (G::VLD * 4)) : OOB_OFFSET;
+    // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load.  Rows beyond the fragment are
+    // redirected to its last row (their probabilities are zero); a tile that does not exist re-reads the first bytes
+    // of the fragment with every lane (one cache line per instruction).
 #pragma unroll
     for (int idx = 0; idx < 8; ++idx) {
-        const int rowoff = ((idx >> 2) * 16 + (idx & 3)) * G::VROW;
+        const int row = min(t0 + q * 4 + (idx >> 2) * 16 + (idx & 3), fv.L - 1);
+        const unsigned long long addr = fv.vbase + (real ? (unsigned long long)(unsigned)row * G::VROW + n * (G::VLD * 4) : 0ull);
 #pragma unroll
         for (int hh = 0; hh < G::NVL; ++hh) {
             if constexpr (G::VLD == 4) {
-                const u32x4 x = __builtin_amdgcn_raw_buffer_load_b128(fv.v, vb + rowoff + hh * 256, 0, HW_KV_AUX);
+                const u32x4 x = __builtin_nontemporal_load(reinterpret_cast<const HW_GLOBAL u32x4*>(addr + hh * 256));
                 t.v[idx][hh * 4 + 0] = x.x;
                 t.v[idx][hh * 4 + 1] = x.y;
                 t.v[idx][hh * 4 + 2] = x.z;
                 t.v[idx][hh * 4 + 3] = x.w;
             } else {
-                const u32x2 x = __builtin_amdgcn_raw_buffer_load_b64(fv.v, vb + rowoff, 0, HW_KV_AUX);
+                const u32x2 x = __builtin_nontemporal_load(reinterpret_cast<const HW_GLOBAL u32x2*>(addr));
                 t.v[idx][0] = x.x;
                 t.v[idx][1] = x.y;
             }
@@ -385,7 +392,6 @@ template <> struct Chunk<F16> {
     }
 };
 
-#define HW_GLOBAL __attribute__((address_space(1)))
 
 // What each wave of a workgroup hands over at the end (row stride padded so that rows land in different banks).
 template <int ROWS, int EV>
