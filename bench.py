@@ -31,8 +31,8 @@ METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 worke
 
 # HBM bytes per launch of the attention kernel measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in
 # separate runs, each scaled by what the same counter reads for the 256 MiB copy kernel this script launches:
-# 0.5 for FETCH_SIZE, 1.0 for WRITE_SIZE): 51.78 MB fetched + 3.03 MB written.  Workloads not measured: None.
-MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_810_000}
+# 0.5 for FETCH_SIZE, 1.0 for WRITE_SIZE): 51.83 MB fetched + 3.03 MB written.  Workloads not measured: None.
+MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_860_000}
 # the same for hw::paged_attention_kernel at the default paged workload (4 x 12528 tokens, blocks of 16): 205.69 MB + 0.67 MB
 MEASURED_PAGED_TRAFFIC_BYTES = {(12528, 16): 206_360_000}
 
