@@ -47,8 +47,9 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
     ap.add_argument("--ring-mb", type=int, default=640)
-    ap.add_argument("--workload", choices=["fragments", "paged"], default="fragments",
-                    help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape")
+    ap.add_argument("--workload", choices=["fragments", "paged", "varlen"], default="fragments",
+                    help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape; "
+                         "varlen = hogwild_varlen_paged_sdpa on the same cache with 1 / 8 / 32 / 64 query tokens per sequence")
     ap.add_argument("--seq-len", type=int, default=12528, help="paged workload: tokens per sequence")
     ap.add_argument("--block-size", type=int, default=16, help="paged workload: tokens per cache block")
     return ap.parse_args()
@@ -89,7 +90,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
-    if args.workload == "paged":
+    if args.workload in ("paged", "varlen"):
         bench_paged(args, dev)
         return
 
@@ -309,11 +310,23 @@ def bench_paged(args, dev):
     kc = torch.randn((NB, Hkv, bs, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
     vc = torch.randn((NB, Hkv, bs, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
     perm = torch.randperm(NB, generator=torch.Generator().manual_seed(8)).to(torch.int32)
-    q = torch.randn((F, W, Hq, S, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
-    loc = torch.full((F, W, S), L - 1, dtype=torch.int32, device=dev)
-    fl = torch.full((F,), L, dtype=torch.int32, device=dev)
-    out = torch.empty((W, Hq, S, D), dtype=torch.bfloat16, device=dev)
-    lse = torch.empty((W, Hq, S), dtype=torch.float32, device=dev)
+    varlen = args.workload == "varlen"
+    cu = None
+    if varlen:   # packed queries: the last 1 / 8 / 32 / 64 positions of the four sequences (causal)
+        q_lens = [1, 8, 32, 64]
+        T = sum(q_lens)
+        cu = torch.tensor([0] + [sum(q_lens[:i + 1]) for i in range(W)], dtype=torch.int32, device=dev)
+        q = torch.randn((F, T, Hq, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        loc = torch.cat([torch.arange(L - n, L, dtype=torch.int32) for n in q_lens]).reshape(F, T).to(dev)
+        fl = torch.full((F, W), L, dtype=torch.int32, device=dev)
+        out = torch.empty((T, Hq, D), dtype=torch.bfloat16, device=dev)
+        lse = torch.empty((T, Hq), dtype=torch.float32, device=dev)
+    else:
+        q = torch.randn((F, W, Hq, S, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        loc = torch.full((F, W, S), L - 1, dtype=torch.int32, device=dev)
+        fl = torch.full((F,), L, dtype=torch.int32, device=dev)
+        out = torch.empty((W, Hq, S, D), dtype=torch.bfloat16, device=dev)
+        lse = torch.empty((W, Hq, S), dtype=torch.float32, device=dev)
     scale = 1.0 / math.sqrt(D)
     problems, tables = [], []
     ws = None
@@ -321,13 +334,13 @@ def bench_paged(args, dev):
         bt = perm[i * W * nblk:(i + 1) * W * nblk].reshape(W, nblk).contiguous().to(dev)
         tables.append(bt)
         pr = _lib.PagedProblem(q=q, locations=loc, fragment_lengths=fl, key_cache=kc, value_cache=vc, block_table=bt,
-                               scale=scale, out=out, lse=lse, splits=args.splits)
+                               scale=scale, out=out, lse=lse, splits=args.splits, cu_seqlens_q=cu)
         if ws is None:
             ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
         pr.set_workspace(ws)
         problems.append(pr)
     plan = _lib.paged_plan(W=W, Hq=Hq, Hkv=Hkv, Ev=D, block_size=bs, max_blocks=nblk, num_cus=_lib.lib.hw_device_cus(), S=S,
-                           splits=args.splits)
+                           splits=args.splits, total_q=(q.size(1) if varlen else None))
     K, Wm = args.steps, args.warmup
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -382,15 +395,16 @@ def bench_paged(args, dev):
     value = kv_bytes / (graph_us * 1e-6) / 1e9
     achieved = kv_bytes / (kern_us * 1e-6) / 1e9
     result = {
-        "metric": "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 sequences, paged KV cache",
+        "metric": "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 sequences, paged KV cache"
+                  + (", packed variable-length queries" if varlen else ""),
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": Wm,
         "ms_per_step": round(graph_us * 1e-3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"paged decode: W={W} sequences x {L} tokens, S={S}, Hq={Hq} Hkv={Hkv} D={D} bf16, "
-                               f"block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
+        "config": {"workload": (f"varlen paged: W={W} sequences x {L} tokens, query tokens per sequence 1/8/32/64, " if varlen else
+                                f"paged decode: W={W} sequences x {L} tokens, S={S}, ") + f"Hq={Hq} Hkv={Hkv} D={D} bf16, block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": MEASURED_PAGED_TRAFFIC_BYTES.get((L, bs)),
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None if varlen else MEASURED_PAGED_TRAFFIC_BYTES.get((L, bs)),
                      "kernel": "hw::paged_attention_kernel",
                      "kernel_us_avg": round(kern_us, 3),
                      "timing": "two HIP events around a graph replay of K attention-kernel launches (merge stage off), divided by K"},
@@ -405,7 +419,11 @@ def bench_paged(args, dev):
         t_all = time.perf_counter()
         while len(ts) < 5 and (time.perf_counter() - t_all) < 30.0:
             t0 = time.perf_counter()
-            po.paged_sdpa(qn, loc.cpu().numpy(), fl.cpu().numpy(), kn, vn, tables[0].cpu().numpy(), scale, dtype=np_f32())
+            if varlen:
+                po.varlen_paged_sdpa(qn, loc.cpu().numpy(), fl.cpu().numpy(), kn, vn, tables[0].cpu().numpy(), cu.cpu().numpy(), scale,
+                                     dtype=np_f32())
+            else:
+                po.paged_sdpa(qn, loc.cpu().numpy(), fl.cpu().numpy(), kn, vn, tables[0].cpu().numpy(), scale, dtype=np_f32())
             ts.append(time.perf_counter() - t0)
         med = sorted(ts)[len(ts) // 2]
         cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)

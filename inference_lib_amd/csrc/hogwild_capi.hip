@@ -292,10 +292,20 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     plan->row_groups = (int)items;
     int splits = p->splits;
     if (splits <= 0) {
-        const long long target = num_cus;   // the paged kernels are built for one workgroup per CU
-        long long s = target / ((long long)p->Hkv * items);
-        // at the longest sequence the table allows, every wave should still have at least one tile
-        const long long by_work = ((long long)p->block_size * p->max_blocks + hw::TILE * hw::NWAVES - 1) / (hw::TILE * hw::NWAVES);
+        // The paged kernels run one workgroup per CU.  Few (kv head, row group) pairs: split until every CU has
+        // one workgroup.  More pairs than half the CUs: the chip is oversubscribed anyway, and about three
+        // workgroups per CU even out the tail between sequences of different length (measured best on packed
+        // variable-length queries) -- there a wave keeps at least four tiles.
+        const long long pairs = (long long)p->Hkv * items;
+        const long long tiles = ((long long)p->block_size * p->max_blocks + hw::TILE - 1) / hw::TILE;
+        long long s, by_work;
+        if (2 * pairs <= num_cus) {
+            s = num_cus / pairs;
+            by_work = (tiles + hw::NWAVES - 1) / hw::NWAVES;
+        } else {
+            s = (3LL * num_cus + pairs - 1) / pairs;
+            by_work = tiles / (4 * hw::NWAVES);
+        }
         if (s > by_work) s = by_work;
         splits = (int)s;
     }

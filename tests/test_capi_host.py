@@ -232,6 +232,12 @@ def test_paged_plan_invariants():
     # variable length: the row-group count is an upper bound over every way of cutting total_q into W sequences
     pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700)
     assert pl.rows == 3500 and pl.row_groups >= 8 + 3500 // 32 and pl.workgroups == 8 * pl.row_groups * pl.splits
+    # more (kv head, row group) pairs than half the CUs: about three workgroups per CU on long sequences, no
+    # splitting at all on short ones or when the pairs alone oversubscribe the chip that far
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
+    assert pl.row_groups == 20 and pl.splits == 5 and 3 * 256 <= pl.workgroups < 4 * 256
+    assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=30, num_cus=256, total_q=105).splits == 1
+    assert L.paged_plan(W=64, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=640).splits == 1
     # explicit split factor is honoured (capped at 64)
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=5).splits == 5
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=500).splits == 64
