@@ -77,16 +77,35 @@ constexpr float NEG_BIG = -1.0e30f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// max over the four lanes {l, l^16, l^32, l^48}: the four quarter-waves hold different tokens of one row
+// Reductions over the four lanes {l, l^16, l^32, l^48}: the four quarter-waves hold different tokens of one row.
+// v_permlane32_swap / v_permlane16_swap exchange half-waves / 16-lane rows between two registers; applied to two
+// copies of a value they leave "mine" in one register and "my partner's" in the other, in every lane, without the
+// trip through the LDS crossbar that a generic shuffle takes.
+__device__ __forceinline__ void quarter_pairs(float v, int step, float& a, float& b) {
+    const u32 x = __float_as_uint(v);
+    if (step == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(x, x, false, false);
+        a = __uint_as_float(r[0]);
+        b = __uint_as_float(r[1]);
+    } else {
+        const auto r = __builtin_amdgcn_permlane16_swap(x, x, false, false);
+        a = __uint_as_float(r[0]);
+        b = __uint_as_float(r[1]);
+    }
+}
 __device__ __forceinline__ float quarter_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16, 64));
-    v = fmaxf(v, __shfl_xor(v, 32, 64));
-    return v;
+    float a, b;
+    quarter_pairs(v, 32, a, b);
+    v = fmaxf(a, b);
+    quarter_pairs(v, 16, a, b);
+    return fmaxf(a, b);
 }
 __device__ __forceinline__ float quarter_sum(float v) {
-    v += __shfl_xor(v, 16, 64);
-    v += __shfl_xor(v, 32, 64);
-    return v;
+    float a, b;
+    quarter_pairs(v, 32, a, b);
+    v = a + b;
+    quarter_pairs(v, 16, a, b);
+    return a + b;
 }
 
 // token (relative to the tile start) held in reduction slot `idx` (0..7) of quarter-wave `q`:
