@@ -204,15 +204,21 @@ def main():
         with torch.cuda.graph(g_b, stream=stream):
             for i in range(K):
                 _lib.build_inputs(pos_end, S, inv, table_dtype=tdt if tdt != torch.float32 else None)
+        # what one layer of a decode step launches: key rotation + append, then attention and merge (cold ring)
+        g_c = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_c, stream=stream):
+            for i in range(K):
+                _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck)
+                problems[i % nring].run()
         side = []
-        for gr in (g_a, g_b):
+        for gr in (g_a, g_b, g_c):
             gr.replay()
             torch.cuda.synchronize()
             t0 = time.perf_counter()
             gr.replay()
             torch.cuda.synchronize()
             side.append((time.perf_counter() - t0) / K * 1e6)
-        append_us, build_us = side
+        append_us, build_us, layer_us = side
 
         # ---------------- plain streaming read of the whole ring (achievable HBM rate) ----------------
         big = torch.empty(int(args.ring_mb * 1e6) // 16 * 16, dtype=torch.uint8, device=dev)
@@ -284,6 +290,7 @@ def main():
             "stream_read_GBps": round(stream_gbs, 1),
             "rope_append_us_per_call": round(append_us, 3),
             "build_inputs_us_per_call": round(build_us, 3),
+            "append_plus_attention_us_per_layer": round(layer_us, 3),
             "timing": "K steps replayed as one HIP graph, wall clock between device synchronisations",
         },
     }
