@@ -449,7 +449,11 @@ __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Excha
     __syncthreads();
     HW_MARK(4);
     HW_GLOBAL float* dst = part_o + part * EV;
-    for (int idx = tid * 4; idx < nrows * EV; idx += NTHREADS * 4) {
+    constexpr int PASSES = (RB * 16 * EV + NTHREADS * 4 - 1) / (NTHREADS * 4);
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {   // fixed trip count: the LDS reads of all passes can be in flight together
+        const int idx = tid * 4 + ps * NTHREADS * 4;
+        if (idx >= nrows * EV) break;
         const int rr = idx / EV, e = idx - rr * EV;
         float mm = ex.m[0][rr];
 #pragma unroll
