@@ -12,16 +12,18 @@ Nothing in the product package imports this module.  It restates, in numpy:
 The rotary embedding module itself lives in the `transformers` dependency of the reference (Qwen2RotaryEmbedding and
 its siblings; the reference pins no version).  Its published algorithm is restated in `rotary_tables`:
 freqs = position.float() * inv_freq.float(); emb = cat(freqs, freqs); cos = emb.cos() * attention_scaling, cast to the
-dtype of the activations.
+dtype of the activations.  Where `transformers` is installed the pins also run against its Qwen2RotaryEmbedding and
+apply_rotary_pos_emb directly.
 
 Pinning status (tests/test_cache_oracle_pins.py):
   pos_end_from_orders ... pinned: closed-form sums; consistency with hogwild_oracle.locations_from_order.
   rotary_tables ......... pinned: equals hogwild_oracle.rope_tables (itself pinned) for inv_freq = base^(-2i/D);
-                          torch.cos/sin in float32 for the fp32 arithmetic; bf16/fp16 rounding via torch casts.
+                          torch.cos/sin in float32 for the fp32 arithmetic; bf16/fp16 rounding via torch casts;
+                          the installed transformers' Qwen2RotaryEmbedding.
   rope_keys ............. pinned: closed-form rotation per element pair; norm preservation; q.k after rotating both
                           sides depends only on the position difference (with the query rotation pinned separately
                           against the reference's rope_cpu); eager rounding order against torch's own tensor
-                          arithmetic in bf16 / fp16 / fp32 on the CPU.
+                          arithmetic in bf16 / fp16 / fp32 on the CPU; transformers' apply_rotary_pos_emb bit for bit.
   append_left_masked .... pinned: torch.cat of the unmasked tails.
   merge_rerotate ........ pinned: rotating keys of position p by a further t equals rotating the raw keys by p + t.
 The reference ships no tests, fixtures or golden vectors for these steps.

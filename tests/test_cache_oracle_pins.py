@@ -144,3 +144,44 @@ def test_merge_rerotation_composes_positions():
     assert np.allclose(merged, direct, atol=5e-5)
     # and it is NOT the identity or a rotation by another offset
     assert np.abs(merged - stored).max() > 0.1
+
+
+# ---------------------------------------------------------------------------------------------- the model library itself
+def test_rotary_tables_match_the_model_librarys_rotary_embedding():
+    """rotary_tables against the rotary embedding module of the installed `transformers` (the module the reference
+    calls, python/hogwild/attention.py:191), for fp32 and bf16 activations and large positions."""
+    transformers = pytest.importorskip("transformers")
+    from transformers import Qwen2Config
+    from transformers.models.qwen2.modeling_qwen2 import Qwen2RotaryEmbedding
+    cfg = Qwen2Config(vocab_size=16, hidden_size=256, intermediate_size=64, num_hidden_layers=1, num_attention_heads=2,
+                      num_key_value_heads=1, max_position_embeddings=4096)
+    rot = Qwen2RotaryEmbedding(cfg)
+    pos = torch.tensor([[0, 1, 2, 77, 4095, 31000]])
+    inv = rot.inv_freq.numpy()
+    for tdt, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16"), (torch.float16, "f16")):
+        cos, sin = rot(torch.zeros(1, 6, 256, dtype=tdt), pos)
+        assert cos.dtype == tdt
+        c, s = co.rotary_tables(pos.numpy(), inv, float(rot.attention_scaling), name)
+        wc, ws = cos.float().numpy(), sin.float().numpy()
+        if name == "f32":
+            assert np.abs(c - wc).max() <= 1.2e-7 and np.abs(s - ws).max() <= 1.2e-7
+        else:       # identical after rounding except where the fp32 values straddle a rounding boundary
+            assert np.mean(c == wc) > 0.995 and np.mean(s == ws) > 0.995
+            assert np.abs(c - wc).max() <= 2 ** -8 and np.abs(s - ws).max() <= 2 ** -8
+
+
+def test_key_rotation_matches_the_model_librarys_apply_rotary_pos_emb():
+    transformers = pytest.importorskip("transformers")
+    from transformers.models.qwen2.modeling_qwen2 import apply_rotary_pos_emb
+    D = 64
+    g = torch.Generator().manual_seed(3)
+    for tdt, name in ((torch.float32, "f32"), (torch.bfloat16, "bf16"), (torch.float16, "f16")):
+        k = torch.randn((2, 3, 5, D), generator=g).to(tdt)
+        pos = torch.tensor([[3, 4, 5, 6, 7], [100, 101, 102, 103, 104]])
+        ang = pos.float()[..., None] * torch.from_numpy(inv_freq(D))
+        emb = torch.cat([ang, ang], -1)
+        cos, sin = emb.cos().to(tdt), emb.sin().to(tdt)
+        _, want = apply_rotary_pos_emb(k, k, cos, sin)            # unsqueezes the tables over the head dimension
+        got = co.rope_keys(k.double().numpy(), cos.double().numpy()[:, None], sin.double().numpy()[:, None], storage=name,
+                           cs_storage=name, mode="eager")
+        assert np.array_equal(got, want.double().numpy())
