@@ -51,8 +51,25 @@ class SegmentCache:
     def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
         return self.lengths[layer_idx or 0]
 
+    def reserve(self, layer_idx: int, n_new: int) -> None:
+        """Room for n_new more tokens in one layer's buffers.  A full segment moves into buffers of twice the size (the
+        transformers caches of the reference grow by torch.cat on every update); the copy is the only reallocation
+        a segment ever sees, and the capacity becomes the new row distance between its kv heads."""
+        need = self.lengths[layer_idx] + int(n_new)
+        cap = self.k[layer_idx].size(1)
+        if need <= cap:
+            return
+        new_cap = max(need, 2 * cap)
+        for bufs in (self.k, self.v):
+            old = bufs[layer_idx]
+            grown = torch.empty((old.size(0), new_cap, old.size(2)), dtype=old.dtype, device=old.device)
+            grown[:, : self.lengths[layer_idx]].copy_(old[:, : self.lengths[layer_idx]])
+            bufs[layer_idx] = grown
+        self.capacity = max(self.capacity, new_cap)
+
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int, cache_kwargs: Optional[Dict[str, Any]] = None):
         """Append [1, Hkv, n, D] keys (already rotated) and values; returns the views of the grown segment."""
+        self.reserve(layer_idx, key_states.size(2))
         _lib.rope_append(key_states, value_states, [self.k[layer_idx]], [self.v[layer_idx]], [self.lengths[layer_idx]])
         self.lengths[layer_idx] += key_states.size(2)
         return self.key_cache[layer_idx], self.value_cache[layer_idx]
@@ -109,6 +126,8 @@ class HogwildCache:
         S = key_states.size(2)
         n_new = [S] * W if mask is None else [int(x) for x in torch.sum(mask, dim=1).tolist()]   # left masking, :149-155
         segs = self.write_to
+        for s, n in zip(segs, n_new):
+            s.reserve(layer_idx, n)
         _lib.rope_append(key_states, value_states, [s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs],
                          [s.lengths[layer_idx] for s in segs], cosines=cosines, sines=sines, n_new=n_new, mode=mode)
         for s, n in zip(segs, n_new):

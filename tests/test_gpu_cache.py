@@ -274,3 +274,19 @@ def test_merge_caches_rerotates_and_appends(dtype):
         else:
             ulp = 2.0 ** -6 if dtype == "bf16" else 2.0 ** -9
             assert np.abs(got_k[:, 77:] - want).max() <= ulp and np.mean(got_k[:, 77:] == want) > 0.99
+
+
+def test_segment_grows_when_full():
+    """A segment that runs out of room moves into buffers of twice the size; contents and later appends are unaffected."""
+    from inference_lib_amd.cache import SegmentCache
+    dev = torch.device("cuda:0")
+    seg = SegmentCache(2, 2, 64, 3, dtype=torch.float16, device=dev)
+    g = torch.Generator().manual_seed(0)
+    parts_k = [torch.randn((1, 2, n, 64), generator=g).half().to(dev) for n in (2, 2, 5, 1)]
+    parts_v = [torch.randn((1, 2, n, 64), generator=g).half().to(dev) for n in (2, 2, 5, 1)]
+    for pk, pv in zip(parts_k, parts_v):
+        print("append", pk.size(2), "to a segment of", seg.get_seq_length(1), "capacity", seg.k[1].size(1), flush=True)
+        seg.update(pk, pv, 1)
+    torch.cuda.synchronize()
+    assert seg.get_seq_length(1) == 10 and seg.get_seq_length(0) == 0 and seg.k[1].size(1) >= 10 and seg.k[0].size(1) == 3
+    assert torch.equal(seg.key_cache[1], torch.cat(parts_k, dim=2)) and torch.equal(seg.value_cache[1], torch.cat(parts_v, dim=2))
