@@ -294,3 +294,47 @@ def test_paged_torch_ops_match_c_abi_and_raise_loudly():
                                      torch.zeros((1, 2), dtype=torch.int32, device=dev), 1.0)
     with pytest.raises(RuntimeError, match="dtype"):
         torch.ops.libhogatt.hogwild_paged_sdpa(out.new_zeros((3, 10, 2, 128)), 1.0, d["loc"], d["q"].float(), d["fl"], d["kc"], d["vc"], d["bt"])
+
+
+def test_paged_cache_larger_than_4_gib():
+    """Caches of 5 GiB each: cache rows beyond the first 4 GiB are reached only if the row address is formed in 64 bits,
+    in the attention kernel and in copy_to_blocks alike.  Closed form instead of the oracle: all keys of the sequence
+    are zero except the newest, appended through copy_to_blocks into the block with the highest id and a large multiple
+    of the query, so the output must be exactly that token's value row."""
+    from inference_lib_amd import _lib
+    dev = torch.device("cuda:0")
+    Hkv, bs, D = 2, 16, 128
+    NB = (5 << 30) // (Hkv * bs * D * 2)              # blocks in a 5 GiB bf16 cache
+    kc = torch.zeros((NB, Hkv, bs, D), dtype=torch.bfloat16, device=dev)
+    vc = torch.zeros((NB, Hkv, bs, D), dtype=torch.bfloat16, device=dev)
+    L = 100                                            # tokens before the append: blocks 0..6 of the table
+    bt = torch.tensor([[NB - 2, 5, NB // 2, NB - 7, 11, NB - 3, NB - 1, NB - 4]], dtype=torch.int32, device=dev)
+    g = torch.Generator().manual_seed(23)
+    for b in bt[0, :7].tolist():                       # random values in the blocks the sequence already occupies
+        vc[b] = torch.randn((Hkv, bs, D), generator=g).to(torch.bfloat16).to(dev)
+    q = torch.randn((1, 1, 4, 1, D), generator=g).to(torch.bfloat16).to(dev)            # [F, W, Hq, S, D], GQA 2
+    k_new = torch.stack([4.0 * q[0, 0, 0, 0].float(), 4.0 * q[0, 0, 2, 0].float()])[None, :, None, :].to(torch.bfloat16)   # [1, Hkv, 1, D]
+    v_new = torch.randn((1, Hkv, 1, D), generator=g).to(torch.bfloat16).to(dev)
+    seq = torch.tensor([L], dtype=torch.int32, device=dev)
+    print(f"copy_to_blocks into block {NB - 1} of {NB}", flush=True)
+    _lib.copy_to_blocks(k_new, v_new, kc, vc, bt, seq)                                   # position 100 = row 4 of table entry 6 = block NB-1
+    torch.cuda.synchronize()
+    assert torch.equal(kc[NB - 1, :, 4], k_new[0, :, 0]) and torch.equal(vc[NB - 1, :, 4], v_new[0, :, 0])
+    assert int((kc != 0).any(dim=-1).sum()) == Hkv                                       # nothing else was written
+    out = torch.full((1, 4, 1, D), float("nan"), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((1, 4, 1), dtype=torch.float32, device=dev)
+    loc = torch.tensor([[[L]]], dtype=torch.int32, device=dev)
+    fl = torch.tensor([L + 1], dtype=torch.int32, device=dev)
+    print("paged attention over blocks on both sides of the 4 GiB line", flush=True)
+    _lib.PagedProblem(q=q, locations=loc, fragment_lengths=fl, key_cache=kc, value_cache=vc, block_table=bt, scale=D ** -0.5,
+                      out=out, lse=lse).run()
+    torch.cuda.synchronize()
+    for h in (0, 2):                                   # the heads whose query the new key is a multiple of
+        assert torch.equal(out[0, h, 0], v_new[0, h // 2, 0])
+    # and a second token, in the middle of the sequence (table entry 3 = block NB-7, beyond 4 GiB as well)
+    kc[NB - 1, :, 4] = 0
+    kc[NB - 7, 1, 9] = k_new[0, 1, 0]                  # position 3 * 16 + 9 = 57, kv head 1
+    _lib.PagedProblem(q=q, locations=loc, fragment_lengths=fl, key_cache=kc, value_cache=vc, block_table=bt, scale=D ** -0.5,
+                      out=out, lse=lse).run()
+    torch.cuda.synchronize()
+    assert torch.equal(out[0, 2, 0], vc[NB - 7, 1, 9])

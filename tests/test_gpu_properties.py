@@ -132,6 +132,42 @@ def test_long_fragment_many_tiles_per_workgroup(oracle):
     assert_close("lse", lse, l_ref, TOL["f16"])
 
 
+def test_fragment_at_the_32_bit_offset_limit():
+    """The longest fragment the byte-offset arithmetic allows (just under 2^31 bytes per kv head, 8.39 M tokens of
+    bf16 at head dim 128).  Closed form instead of the oracle: all keys are zero except one, which is a large multiple
+    of the query, so the softmax is that token alone and the output must be exactly its value row -- at the last
+    token (highest offsets), in the middle, and at the first.  One token more is refused."""
+    from inference_lib_amd import _lib
+    dev = _dev()
+    L, E = 8_388_000, 128
+    g = torch.Generator().manual_seed(17)
+    q = torch.randn((1, 1, 1, E), generator=g).to(torch.bfloat16).to(dev)
+    K = torch.zeros((1, L, E), dtype=torch.bfloat16, device=dev)
+    V = torch.empty((1, L, E), dtype=torch.bfloat16, device=dev).normal_(generator=torch.Generator(device=dev).manual_seed(1))
+    loc = torch.tensor([[[L - 1]]], dtype=torch.int32, device=dev)
+    cos = torch.ones((1, 1, 1, E), dtype=torch.float32, device=dev)
+    sin = torch.zeros((1, 1, 1, E), dtype=torch.float32, device=dev)
+    out = torch.empty((1, 1, 1, E), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((1, 1, 1), dtype=torch.float32, device=dev)
+    scale = E ** -0.5
+    for idx in (L - 1, 5_000_001, 0):
+        print(f"peak at token {idx} of {L}", flush=True)
+        K.zero_()
+        K[0, idx] = (4.0 * q[0, 0, 0].float()).to(torch.bfloat16)
+        _lib.Problem(q=q, locations=loc, keys=[K], values=[V], scale=scale, out=out, cosines=cos, sines=sin, lse=lse).run()
+        torch.cuda.synchronize()
+        score = float((q[0, 0, 0].float() * K[0, idx].float()).sum()) * scale
+        assert score > 30
+        assert torch.equal(out[0, 0, 0], V[0, idx])
+        assert abs(float(lse) - score) <= 1e-3          # the other 8.4 M tokens weigh e^(16 - score)
+    del K, V
+    too_long = 0x7fff0000 // (E * 2)                     # first length whose byte size reaches the limit
+    K = torch.zeros((1, too_long, E), dtype=torch.bfloat16, device=dev)
+    with pytest.raises(_lib.HogwildError) as ei:
+        _lib.Problem(q=q, locations=loc, keys=[K], values=[K], scale=scale, out=out, cosines=cos, sines=sin, lse=lse).run()
+    assert ei.value.status == -3
+
+
 def test_two_stages_equal_the_fused_call():
     from inference_lib_amd import cases
     cd = cases.baseline_case(2).to(_dev())
