@@ -35,6 +35,9 @@ METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 worke
 MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_860_000}
 # the same for hw::paged_attention_kernel at the default paged workload (4 x 12528 tokens, blocks of 16): 205.69 MB + 0.67 MB
 MEASURED_PAGED_TRAFFIC_BYTES = {(12528, 16): 206_360_000}
+# packed variable-length workload on the same cache: 383.36 MB fetched (1.87 x the algorithmic bytes: L2 and the Infinity
+# Cache serve most but not all of the 20 row groups' repeats) + 10.92 MB of split-K partials written
+MEASURED_VARLEN_TRAFFIC_BYTES = {(12528, 16): 394_280_000}
 
 
 def parse_args():
@@ -411,7 +414,7 @@ def bench_paged(args, dev):
                                 f"paged decode: W={W} sequences x {L} tokens, S={S}, ") + f"Hq={Hq} Hkv={Hkv} D={D} bf16, block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None if varlen else MEASURED_PAGED_TRAFFIC_BYTES.get((L, bs)),
+                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": (MEASURED_VARLEN_TRAFFIC_BYTES if varlen else MEASURED_PAGED_TRAFFIC_BYTES).get((L, bs)),
                      "kernel": "hw::paged_attention_kernel",
                      "kernel_us_avg": round(kern_us, 3),
                      "timing": "two HIP events around a graph replay of K attention-kernel launches (merge stage off), divided by K"},
