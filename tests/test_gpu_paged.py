@@ -338,3 +338,66 @@ def test_paged_cache_larger_than_4_gib():
                       out=out, lse=lse).run()
     torch.cuda.synchronize()
     assert torch.equal(out[0, 2, 0], vc[NB - 7, 1, 9])
+
+
+def test_paged_decode_steps_replayed_from_one_graph():
+    """A whole paged decode step (append the new token with copy_to_blocks, advance the sequence lengths, attend) is
+    captured once and replayed while the sequences grow: lengths, locations and block tables live in device memory, the
+    library allocates nothing and records no memset.  Every replay is checked against the oracle on the state it saw,
+    with eager work and synchronisations between the replays."""
+    from inference_lib_amd import _lib
+    from oracle import paged_oracle as po
+    dev = torch.device("cuda:0")
+    W, Hq, Hkv, D, bs, mb = 3, 8, 2, 128, 16, 12
+    seq0 = [37, 150, 16]
+    c = build_paged("bf16", 1, W, Hq, Hkv, D, bs, mb, seq_lens=seq0, S=1, seed=41, poison=False)
+    kc, vc, bt = c["kc"].to(dev), c["vc"].to(dev), c["bt"].to(dev)
+    for w in range(W):      # every table entry a sequence can grow into must be a real block
+        bt[w] = torch.arange(w * mb, (w + 1) * mb, dtype=torch.int32, device=dev)
+    for w in range(W):
+        for p in range(seq0[w]):
+            kc[bt[w, p // bs], :, p % bs] = torch.randn((Hkv, D), generator=torch.Generator().manual_seed(1000 * w + p)).to(torch.bfloat16).to(dev)
+            vc[bt[w, p // bs], :, p % bs] = torch.randn((Hkv, D), generator=torch.Generator().manual_seed(5000 + 1000 * w + p)).to(torch.bfloat16).to(dev)
+    seq = torch.tensor(seq0, dtype=torch.int32, device=dev)
+    loc = torch.zeros((1, W, 1), dtype=torch.int32, device=dev)
+    fl = torch.tensor([bs * mb], dtype=torch.int32, device=dev)        # visibility is bounded by the locations alone
+    q = torch.zeros((1, W, Hq, 1, D), dtype=torch.bfloat16, device=dev)
+    k_new = torch.zeros((W, Hkv, 1, D), dtype=torch.bfloat16, device=dev)
+    v_new = torch.zeros((W, Hkv, 1, D), dtype=torch.bfloat16, device=dev)
+    out = torch.empty((W, Hq, 1, D), dtype=torch.bfloat16, device=dev)
+    lse = torch.empty((W, Hq, 1), dtype=torch.float32, device=dev)
+    pr = _lib.PagedProblem(q=q, locations=loc, fragment_lengths=fl, key_cache=kc, value_cache=vc, block_table=bt, scale=c["scale"],
+                           out=out, lse=lse)
+    pr.set_workspace()
+
+    def step():
+        _lib.copy_to_blocks(k_new, v_new, kc, vc, bt, seq)      # position seq[w] of every sequence
+        loc.copy_(seq.view(1, W, 1))                             # the new token sits at the old length ...
+        seq.add_(1)                                              # ... and the sequence is one longer
+        pr.run()
+
+    stream = torch.cuda.Stream()
+    g = torch.Generator().manual_seed(7)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        step()                                                   # warm-up (also a real step)
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+        seq.copy_(torch.tensor(seq0, dtype=torch.int32))         # capture does not execute; start over from the initial state
+        for it in range(6):
+            q.copy_(torch.randn(q.shape, generator=g).to(torch.bfloat16))
+            k_new.copy_(torch.randn(k_new.shape, generator=g).to(torch.bfloat16))
+            v_new.copy_(torch.randn(v_new.shape, generator=g).to(torch.bfloat16))
+            torch.cuda.synchronize()
+            print(f"replay {it}: sequence lengths {seq.tolist()}", flush=True)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert seq.tolist() == [s + it + 1 for s in seq0]
+            want_o, want_l = po.paged_sdpa(np64(q), loc.cpu().numpy(), fl.cpu().numpy(), np64(kc), np64(vc), bt.cpu().numpy(), c["scale"])
+            assert_close("out", out, want_o, TOL["bf16"])
+            assert_close("lse", lse, want_l, TOL["bf16"])
+            for w in range(W):                                   # the appended rows are where the next step expects them
+                p = seq0[w] + it
+                assert torch.equal(kc[bt[w, p // bs], :, p % bs], k_new[w, :, 0])
+            (out.float().sum() + 1).item()                       # eager work between the replays
