@@ -158,6 +158,25 @@ def main():
         torch.cuda.synchronize()
         hot_us = (time.perf_counter() - t0) / K * 1e6
 
+        # ---------------- the same steps with the fragment lengths read from device memory ----------------
+        len_dev = torch.tensor(case.lens, dtype=torch.int32, device=dev)
+        problems_dl = []
+        for keys, vals in ring:
+            pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=out,
+                              cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse, splits=args.splits, len_dev=len_dev)
+            pr.set_workspace(ws)
+            problems_dl.append(pr)
+        graph_dl = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph_dl, stream=stream):
+            for i in range(K):
+                problems_dl[i % nring].run()
+        graph_dl.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph_dl.replay()
+        torch.cuda.synchronize()
+        devlen_us = (time.perf_counter() - t0) / K * 1e6
+
         # ---------------- per-launch duration of the attention kernel (HIP events on its stream) ----------------
         # K launches of the attention kernel alone (merge stage off), replayed as one graph so that the launches
         # follow each other without host submission gaps, bracketed by two HIP events recorded on this stream.
@@ -289,6 +308,7 @@ def main():
             "eager_loop_us_per_step": round(eager_us, 3),
             "kernel_us_median_eager_event_pair": round(kern_us_eager_med, 3),
             "hot_cache_us_per_step": round(hot_us, 3),
+            "device_lengths_us_per_step": round(devlen_us, 3),
             "hot_cache_GBps": round(kv_bytes / (hot_us * 1e-6) / 1e9, 1),
             "stream_read_GBps": round(stream_gbs, 1),
             "rope_append_us_per_call": round(append_us, 3),

@@ -26,6 +26,9 @@
  *                            (locations :173-181, model.rotary_emb + float cast :191-193)
  *   hw_rope_append ......... apply_rotary_pos_emb on the new keys + the per-worker cache update,
  *                            python/hogwild/attention.py:84-90, :313-318, :148-158; and merge_caches, :251-257
+ *   hw_build_inputs_dev, hw_advance_lengths, hw_problem.len_dev, hw_append.len_dev ... no counterpart: the same steps
+ *                            with the segment lengths in device memory, so that a decode step captured as a HIP graph
+ *                            can be replayed while the segments grow
  */
 #ifndef HOGWILD_HIP_H
 #define HOGWILD_HIP_H
@@ -37,7 +40,7 @@
 extern "C" {
 #endif
 
-#define HW_ABI_VERSION 2
+#define HW_ABI_VERSION 3
 #define HW_MAX_FRAGMENTS 32
 #define HW_MAX_SPLITS 256      /* workgroups per kv head */
 
@@ -72,6 +75,11 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   len        HOST array of F lengths (the reference reads the same numbers from the tensor sizes, src/binding.cu:91)
  *   cap        optional HOST array of F row capacities: kv head h of fragment f starts h * cap[f] rows into its
  *              buffers (a segment that grows in place inside a [Hkv, cap, D] allocation).  NULL = packed, cap == len.
+ *   len_dev    optional DEVICE array of F current lengths (hw_fused_attention with RotE == E only).  With it, len[f] is
+ *              the bound the split is planned for and the buffers must hold (cap[f] >= len[f]), and fragment f has
+ *              min(len[f], len_dev[f]) tokens when the kernel runs: a launch captured in a HIP graph stays valid while
+ *              the segments grow up to len[f].  No counterpart in the reference, whose segments are re-allocated by
+ *              torch.cat on every update (python/hogwild/attention.py:148-158).
  *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
@@ -100,6 +108,7 @@ typedef struct hw_problem {
     void* ev_start;
     void* ev_stop;
     const int32_t* cap;
+    const int32_t* len_dev;
 } hw_problem;
 
 /* How a problem is cut into workgroups; filled by hw_plan_debug (host only, no device needed). */
@@ -252,6 +261,20 @@ int hw_copy_to_blocks(const hw_copy_blocks* c, void* stream);
 int hw_build_inputs(int32_t* locations, float* cosines, float* sines, const int32_t* pos_end, const float* inv_freq,
                     float attention_scaling, int round_dtype, int F, int W, int S, int RotE, void* stream);
 
+/*
+ * The same with the lengths in device memory, for decode steps replayed from a HIP graph: pos_end[f][w] is formed in
+ * the kernel as the sum of len_dev over fragment f and everything behind it in worker w's order.
+ *   len_dev    device int32 [F]: current fragment lengths (including this step's new tokens)
+ *   orders     HOST int32 [W, F]: orders[w][i] = the i-th fragment of worker w's order (every fragment once)
+ * F * W <= 768.
+ */
+int hw_build_inputs_dev(int32_t* locations, float* cosines, float* sines, const int32_t* len_dev, const int32_t* orders,
+                        const float* inv_freq, float attention_scaling, int round_dtype, int F, int W, int S, int RotE,
+                        void* stream);
+
+/* len_dev[f] += add[f] for f < F <= HW_MAX_FRAGMENTS (add is a HOST array): the first node of a captured decode step. */
+int hw_advance_lengths(int32_t* len_dev, const int32_t* add, int F, void* stream);
+
 #define HW_ROPE_EAGER 0   /* every product and the sum rounded as an eager tensor expression rounds them: bit-identical to
                              apply_rotary_pos_emb of the reference on the same dtypes */
 #define HW_ROPE_FUSED 1   /* fp32 fused multiply-add, one rounding at the end */
@@ -269,6 +292,9 @@ int hw_build_inputs(int32_t* locations, float* cosines, float* sines, const int3
  *                               python/hogwild/attention.py:252-256)
  *   k_dst / v_dst               HOST arrays of W device pointers to segment buffers [Hkv, cap[w], E|Ev]
  *   dst_len / dst_cap / n_new   HOST arrays of W ints; len + n_new <= cap is checked on the host
+ *   len_dev                     optional DEVICE int32 array of segment lengths.  With it dst_len[w] is an index into it,
+ *                               len_dev[dst_len[w]] is the length of worker w's segment AFTER this append (rows already
+ *                               there = that minus n_new[w]), and an append that would not fit dst_cap[w] is dropped.
  */
 typedef struct hw_append {
     int32_t dtype, cs_dtype, mode;
@@ -285,6 +311,7 @@ typedef struct hw_append {
     const int32_t* dst_len;
     const int32_t* dst_cap;
     const int32_t* n_new;
+    const int32_t* len_dev;
 } hw_append;
 
 int hw_rope_append(const hw_append* a, void* stream);

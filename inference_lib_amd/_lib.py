@@ -27,6 +27,7 @@ EXPORTS = [
     "hw_stream_read", "hw_stream_copy",
     "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
     "hw_paged_sdpa_stages", "hw_copy_to_blocks", "hw_build_inputs", "hw_rope_append",
+    "hw_build_inputs_dev", "hw_advance_lengths",
 ]
 
 
@@ -43,6 +44,7 @@ class HwProblem(C.Structure):
         ("splits", C.c_int32), ("row_blocks", C.c_int32),
         ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p),
         ("cap", C.POINTER(C.c_int32)),
+        ("len_dev", C.c_void_p),
     ]
 
 
@@ -102,6 +104,7 @@ class HwAppend(C.Structure):
         ("cs_w", C.c_int64), ("cs_s", C.c_int64),
         ("k_dst", C.POINTER(C.c_void_p)), ("v_dst", C.POINTER(C.c_void_p)),
         ("dst_len", C.POINTER(C.c_int32)), ("dst_cap", C.POINTER(C.c_int32)), ("n_new", C.POINTER(C.c_int32)),
+        ("len_dev", C.c_void_p),
     ]
 
 
@@ -148,6 +151,9 @@ def _load() -> C.CDLL:
     lib.hw_build_inputs.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_void_p, C.c_float, C.c_int,
                                     C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
     lib.hw_rope_append.argtypes = [C.POINTER(HwAppend), C.c_void_p]
+    lib.hw_build_inputs_dev.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(C.c_int32), C.c_void_p, C.c_float,
+                                        C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_void_p]
+    lib.hw_advance_lengths.argtypes = [C.c_void_p, C.POINTER(C.c_int32), C.c_int, C.c_void_p]
     return lib
 
 
@@ -197,7 +203,7 @@ class Problem:
                  values: Sequence[torch.Tensor], scale: float, out: torch.Tensor,
                  cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
                  rq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                 prerotated: bool = False, splits: int = 0, row_blocks: int = 0):
+                 prerotated: bool = False, splits: int = 0, row_blocks: int = 0, len_dev: Optional[torch.Tensor] = None):
         keys = [_frag3(k) for k in keys]
         values = [_frag3(v) for v in values]
         F = len(keys)
@@ -250,6 +256,10 @@ class Problem:
             if tuple(lse.shape) != (W, Hq, S) or lse.dtype != torch.float32:
                 raise ValueError("lse must be float32 [W, Hq, S]")
             tensors.append(lse)
+        if len_dev is not None:      # current lengths in device memory; the fragment tensors then give the planned bounds
+            if len_dev.dtype != torch.int32 or tuple(len_dev.shape) != (F,):
+                raise ValueError("len_dev must be int32 [F]")
+            tensors.append(len_dev)
         for t in tensors:
             if not t.is_contiguous():
                 raise ValueError("all tensors must be contiguous")
@@ -276,6 +286,7 @@ class Problem:
         p.v = C.cast(self._v, C.POINTER(C.c_void_p))
         p.len = C.cast(self._len, C.POINTER(C.c_int32))
         p.cap = C.cast(self._cap, C.POINTER(C.c_int32))
+        p.len_dev = len_dev.data_ptr() if len_dev is not None else None
         p.splits = int(splits)
         p.row_blocks = int(row_blocks)
         self.p = p
@@ -526,13 +537,57 @@ def build_inputs(pos_end: Sequence[Sequence[int]], S: int, inv_freq: Optional[to
     return loc, cos, sin
 
 
+def build_inputs_dev(len_dev: torch.Tensor, orders: Sequence[Sequence[int]], S: int, inv_freq: Optional[torch.Tensor], *,
+                     attention_scaling: float = 1.0, table_dtype: Optional[torch.dtype] = None, out=None):
+    """build_inputs with the fragment lengths in device memory: len_dev int32 [F] (lengths including this step's new
+    tokens), orders[w] = the fragments in worker w's order.  out = (locations, cosines, sines) to write into (so that a
+    captured graph keeps its addresses), else fresh tensors."""
+    F, W = len_dev.numel(), len(orders)
+    flat = [int(x) for row in orders for x in row]
+    if len(flat) != F * W:
+        raise ValueError("every worker's order must list all F fragments")
+    if len_dev.dtype != torch.int32 or not len_dev.is_contiguous():
+        raise ValueError("len_dev must be contiguous int32 [F]")
+    device = len_dev.device
+    rot = 0 if inv_freq is None else 2 * inv_freq.numel()
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous() or inv_freq.device != device):
+        raise ValueError("inv_freq must be contiguous float32 [RotE/2] on the device of len_dev")
+    if out is None:
+        out = (torch.empty((F, W, S), dtype=torch.int32, device=device), torch.empty((F, W, S, rot), dtype=torch.float32, device=device),
+               torch.empty((F, W, S, rot), dtype=torch.float32, device=device))
+    loc, cos, sin = out
+    if tuple(loc.shape) != (F, W, S) or loc.dtype != torch.int32 or tuple(cos.shape) != (F, W, S, rot) or tuple(sin.shape) != (F, W, S, rot) \
+            or cos.dtype != torch.float32 or sin.dtype != torch.float32 or not (loc.is_contiguous() and cos.is_contiguous() and sin.is_contiguous()):
+        raise ValueError("out must be (int32 [F, W, S], float32 [F, W, S, RotE], float32 [F, W, S, RotE]), contiguous")
+    arr = (C.c_int32 * (F * W))(*flat)
+    rd = HW_F32 if table_dtype is None else _DTYPE_CODE[table_dtype]
+    with torch.cuda.device(device):
+        stream = torch.cuda.current_stream(device).cuda_stream
+        check(lib.hw_build_inputs_dev(loc.data_ptr(), cos.data_ptr(), sin.data_ptr(), len_dev.data_ptr(), arr,
+                                      inv_freq.data_ptr() if inv_freq is not None else None, float(attention_scaling), rd,
+                                      F, W, S, rot, C.c_void_p(stream)), "hw_build_inputs_dev")
+    return loc, cos, sin
+
+
+def advance_lengths(len_dev: torch.Tensor, add: Sequence[int]) -> None:
+    """len_dev[f] += add[f] on the device (add: host numbers)."""
+    F = len_dev.numel()
+    if len_dev.dtype != torch.int32 or not len_dev.is_contiguous() or len(add) != F:
+        raise ValueError("len_dev must be contiguous int32 [F] and add one number per entry")
+    arr = (C.c_int32 * F)(*[int(x) for x in add])
+    with torch.cuda.device(len_dev.device):
+        stream = torch.cuda.current_stream(len_dev.device).cuda_stream
+        check(lib.hw_advance_lengths(len_dev.data_ptr(), arr, F, C.c_void_p(stream)), "hw_advance_lengths")
+
+
 def rope_append(key_states: torch.Tensor, value_states: torch.Tensor, k_dst: Sequence[torch.Tensor], v_dst: Sequence[torch.Tensor],
                 dst_len: Sequence[int], *, cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
-                n_new: Optional[Sequence[int]] = None, mode: int = HW_ROPE_EAGER) -> None:
+                n_new: Optional[Sequence[int]] = None, mode: int = HW_ROPE_EAGER, len_dev: Optional[torch.Tensor] = None) -> None:
     """Rotate key_states [W, Hkv, S, E] with cosines / sines [W, S, RotE] (or [W, 1, RotE]: one row for all tokens) and
     append keys and value_states [W, Hkv, S, Ev] to the segment buffers k_dst[w] / v_dst[w] ([Hkv, cap, E|Ev], contiguous)
     behind their first dst_len[w] rows.  Without cosines the keys are appended as they are.  n_new[w] < S appends only
-    the last n_new[w] tokens of worker w."""
+    the last n_new[w] tokens of worker w.  With len_dev (int32 device tensor of segment lengths) dst_len[w] is an index
+    into it and len_dev[dst_len[w]] the length of worker w's segment after this append."""
     if key_states.dim() != 4 or value_states.dim() != 4 or key_states.shape[:3] != value_states.shape[:3]:
         raise ValueError("key_states / value_states must be [W, Hkv, S, E|Ev]")
     W, Hkv, S, E = key_states.shape
@@ -577,6 +632,12 @@ def rope_append(key_states: torch.Tensor, value_states: torch.Tensor, k_dst: Seq
     nn = (C.c_int32 * W)(*([S] * W if n_new is None else [int(x) for x in n_new]))
     a.k_dst, a.v_dst = C.cast(kp, C.POINTER(C.c_void_p)), C.cast(vp, C.POINTER(C.c_void_p))
     a.dst_len, a.dst_cap, a.n_new = C.cast(ln, C.POINTER(C.c_int32)), C.cast(cp, C.POINTER(C.c_int32)), C.cast(nn, C.POINTER(C.c_int32))
+    if len_dev is not None:
+        if len_dev.dtype != torch.int32 or len_dev.dim() != 1 or not len_dev.is_contiguous() or len_dev.device != key_states.device:
+            raise ValueError("len_dev must be a contiguous int32 vector on the device of the new states")
+        if any(int(x) < 0 or int(x) >= len_dev.numel() for x in dst_len):
+            raise ValueError("with len_dev, dst_len holds indices into it")
+        a.len_dev = len_dev.data_ptr()
     with torch.cuda.device(key_states.device):
         stream = torch.cuda.current_stream(key_states.device).cuda_stream
         check(lib.hw_rope_append(C.byref(a), C.c_void_p(stream)), "hw_rope_append")

@@ -25,11 +25,22 @@ if os.path.exists(_TORCH_EXT):
 
 def hogwild_fused(queries: torch.Tensor, locations: torch.Tensor, keys: List[torch.Tensor], values: List[torch.Tensor],
                   scale: float, fragment_lengths, cosines: torch.Tensor, sines: torch.Tensor, *, rotated_queries, out,
-                  lse: Optional[torch.Tensor] = None):
+                  lse: Optional[torch.Tensor] = None, device_lengths: bool = False):
     """rope + attention in one pass (python/hogwild/attention.py:19-23).  `fragment_lengths` is accepted
     for signature compatibility; the lengths are taken from the fragment tensors, which the reference
     requires to agree with it (src/kernels/kernel_v21.cuh:116-117).  `lse` (float32 [W,Hq,S]) is an
-    addition: natural-log log-sum-exp of the scaled visible logits."""
+    addition: natural-log log-sum-exp of the scaled visible logits.  device_lengths (an addition as well): the
+    fragment tensors give bounds and `fragment_lengths` (int32 [F] in device memory) the current lengths, fragment f
+    having min(size, fragment_lengths[f]) tokens -- for launches captured in a graph while segments grow in place."""
+    if device_lengths:
+        if HAVE_TORCH_OPS and lse is None:
+            torch.ops.libhogatt.hogwild_fused_devlen(out, rotated_queries, scale, locations, queries.contiguous(), fragment_lengths,
+                                                     keys, values, cosines, sines)
+            return out
+        pr = _lib.Problem(q=queries.contiguous(), locations=locations, keys=keys, values=values, scale=scale, out=out,
+                          cosines=cosines, sines=sines, rq=rotated_queries, lse=lse, len_dev=fragment_lengths)
+        pr.run()
+        return out
     if HAVE_TORCH_OPS and lse is None:
         torch.ops.libhogatt.hogwild_fused(out, rotated_queries, scale, locations, queries.contiguous(), fragment_lengths,
                                           keys, values, cosines, sines)

@@ -115,6 +115,76 @@ class HogwildCache:
         self.segments: List[SegmentCache] = []
         self.queries_buffer = None
         self.att_buffer = None
+        self._dev = None        # state of the device-resident-lengths mode, see use_device_lengths
+
+    # ---- lengths in device memory: decode steps that can be captured once and replayed ------------------------------
+    def use_device_lengths(self, headroom: int, new_tokens: int = 1) -> None:
+        """From now on the segment lengths live in a device tensor that every step advances on the device, so a decode
+        step (update_fused + hogwild_fused for every layer) can be captured in a HIP graph once and replayed while the
+        segments grow: nothing about a step depends on host numbers any more.  Every worker appends `new_tokens` tokens
+        per step (no left masking in this mode).  The attention split is planned for lengths up to `headroom` tokens
+        beyond the present ones, and the buffers are grown to hold them now, so a capture is good for
+        headroom // new_tokens steps; call this again to re-plan.  The host-side lengths are not touched by the steps:
+        sync_lengths() reads them back.  No counterpart in the reference, whose segments are re-allocated on every
+        update (attention.py:148-158)."""
+        segments = list(self.cache_structure[0])
+        index = {id(cs): f for f, cs in enumerate(segments)}
+        for seg in segments:
+            if len(set(seg.lengths)) != 1:
+                raise ValueError("all layers of a segment must hold the same number of tokens (call between decode steps)")
+        add = [0] * len(segments)
+        for seg in self.write_to:
+            add[index[id(seg)]] += int(new_tokens)
+        bound = [seg.get_seq_length() + (int(headroom) if add[f] else 0) for f, seg in enumerate(segments)]
+        for f, seg in enumerate(segments):
+            for layer in range(len(seg.k)):
+                seg.reserve(layer, bound[f] - seg.lengths[layer])
+        dev = segments[0].k[0].device
+        self._dev = {
+            "segments": segments, "orders": [[index[id(cs)] for cs in order] for order in self.cache_structure],
+            "write_index": [index[id(seg)] for seg in self.write_to], "add": add, "S": int(new_tokens), "bound": bound,
+            "len_dev": torch.tensor([seg.get_seq_length() for seg in segments], dtype=torch.int32, device=dev),
+            "write_index_dev": torch.tensor([index[id(seg)] for seg in self.write_to], dtype=torch.int64, device=dev),
+            "tables": None,
+        }
+
+    @property
+    def device_lengths(self) -> bool:
+        return self._dev is not None
+
+    def sync_lengths(self) -> None:
+        """Device-resident lengths -> host-side lengths of every segment and layer (synchronises with the device)."""
+        if self._dev is None:
+            return
+        for seg, n in zip(self._dev["segments"], self._dev["len_dev"].tolist()):
+            seg.lengths = [int(n)] * len(seg.lengths)
+
+    def use_host_lengths(self) -> None:
+        """Leave the device-resident-lengths mode (after reading the lengths back)."""
+        self.sync_lengths()
+        self._dev = None
+
+    def _update_dev(self, key_states, value_states, cos, sin, layer_idx, mode) -> CacheStructure:
+        d = self._dev
+        W, S = key_states.size(0), key_states.size(2)
+        if W != len(self.cache_structure) or S != d["S"]:
+            raise ValueError(f"device-resident lengths were set up for {len(self.cache_structure)} workers x {d['S']} new tokens")
+        if layer_idx == 0:
+            _lib.advance_lengths(d["len_dev"], d["add"])                  # lengths including this step's tokens
+            tdt = self.table_dtype if self.table_dtype is not None else key_states.dtype
+            d["tables"] = _lib.build_inputs_dev(d["len_dev"], d["orders"], S, self.inv_freq.to(key_states.device),
+                                                attention_scaling=self.attention_scaling,
+                                                table_dtype=None if tdt == torch.float32 else tdt, out=d["tables"])
+            self.locations, self.cosines, self.sines = d["tables"]
+            self.segments = d["segments"]
+            self.frags = d["len_dev"]
+        segs = self.write_to
+        _lib.rope_append(key_states, value_states, [s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs], d["write_index"],
+                         cosines=cos, sines=sin, mode=mode, len_dev=d["len_dev"])
+        # the fragments as the operator sees them: views up to the planned bounds, current lengths in `frags`
+        keys = [seg.k[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
+        vals = [seg.v[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
+        return CacheStructure(keys=keys, values=vals, cos=self.cosines, sin=self.sines, loc=self.locations, frags=self.frags)
 
     def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
         return self.cache_structure[0][-1].get_seq_length()        # attention.py:133-135
@@ -158,6 +228,10 @@ class HogwildCache:
                cache_kwargs: Optional[Dict[str, Any]] = None) -> CacheStructure:
         """key_states [W, Hkv, S, D] already rotated (the reference rotates them before the call, attention.py:315)."""
         mask = (cache_kwargs or {}).get("mask", None)
+        if self._dev is not None:
+            if mask is not None:
+                raise ValueError("left masking is not available with device-resident lengths")
+            return self._update_dev(key_states, value_states, None, None, layer_idx, _lib.HW_ROPE_EAGER)
         self._append(key_states, value_states, layer_idx, mask, None, None, _lib.HW_ROPE_EAGER)
         return self._structure(key_states, layer_idx)
 
@@ -165,6 +239,10 @@ class HogwildCache:
                      mask: Optional[torch.Tensor] = None, mode: int = _lib.HW_ROPE_EAGER) -> CacheStructure:
         """The same with un-rotated keys and the model's position embeddings cos/sin [W, S, RotE] of the new tokens:
         rotation (attention.py:313-315) and append (:148-158) in one launch."""
+        if self._dev is not None:
+            if mask is not None:
+                raise ValueError("left masking is not available with device-resident lengths")
+            return self._update_dev(key_states, value_states, cos, sin, layer_idx, mode)
         self._append(key_states, value_states, layer_idx, mask, cos, sin, mode)
         return self._structure(key_states, layer_idx)
 
@@ -185,6 +263,12 @@ class HogwildCache:
         nw = len(self.cache_structure)
         assert input_ids.shape[0] == nw, (input_ids.shape, nw)
         S = input_ids.shape[1]
+        if self._dev is not None:      # positions from the lengths in device memory (before this step's append)
+            if attention_mask is not None:
+                raise ValueError("left masking is not available with device-resident lengths")
+            start = self._dev["len_dev"].index_select(0, self._dev["write_index_dev"]).to(torch.int64)
+            pos_ids = start[:, None] + torch.arange(S, dtype=torch.int64, device=input_ids.device)[None, :]
+            return {"input_ids": input_ids, "attention_mask": None, "past_key_values": self, "use_cache": True, "position_ids": pos_ids}
         new = [S] * nw if attention_mask is None else [int(x) for x in torch.sum(attention_mask, dim=1).tolist()]
         ends = torch.tensor([self.cache_structure[w][-1].get_seq_length() + new[w] for w in range(nw)], dtype=torch.int64, device=input_ids.device)
         pos_ids = ends[:, None] - S + torch.arange(S, dtype=torch.int64, device=input_ids.device)[None, :]

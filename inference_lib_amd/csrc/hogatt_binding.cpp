@@ -15,7 +15,8 @@
 //     of a host-to-device copy per call (src/binding.cu:77-103);
 //   * `fragment_lengths` is accepted for schema compatibility; the lengths are read from the fragment sizes,
 //     which the reference requires to be equal to it (src/kernels/kernel_v21.cuh:116-117);
-//   * `hogwild_fused_lse` / `hogwild_sdpa_lse` additionally return the log-sum-exp per query row.
+//   * `hogwild_fused_lse` / `hogwild_sdpa_lse` additionally return the log-sum-exp per query row;
+//   * `hogwild_fused_devlen` takes the current fragment lengths from `fragment_lengths` in device memory.
 
 #include <ATen/Tensor.h>
 #include <ATen/ops/empty.h>
@@ -232,6 +233,22 @@ void hogwild_fused(at::Tensor& out, at::Tensor& rq, double scale, const at::Tens
     run(u, out, true);
 }
 
+// Addition: the fused operator with `fragment_lengths` (int32 [F] in device memory) as the CURRENT lengths and the
+// fragment tensors' sizes as bounds: fragment f has min(size, fragment_lengths[f]) tokens when the kernel runs, so a
+// captured launch stays valid while segments grow inside their buffers.  (The reference reads the lengths from this
+// tensor as well, src/kernels/kernel_v21.cuh:116-117, but needs them equal to the sizes.)
+void hogwild_fused_devlen(at::Tensor& out, at::Tensor& rq, double scale, const at::Tensor& locations, const at::Tensor& queries,
+                          const at::Tensor& fragment_lengths, const std::vector<at::Tensor>& key_fragments,
+                          const std::vector<at::Tensor>& value_fragments, const at::Tensor& cosines, const at::Tensor& sines) {
+    Unpacked u;
+    unpack_common(u, out, scale, locations, queries, fragment_lengths, key_fragments, value_fragments, false, false);
+    TORCH_CHECK(fragment_lengths.scalar_type() == at::kInt && fragment_lengths.is_contiguous() && fragment_lengths.device() == out.device(),
+                "libhogatt: fragment_lengths must be contiguous int32 on the output's device");
+    attach_rotation(u, out, rq, cosines, sines);
+    u.p.len_dev = fragment_lengths.const_data_ptr<int32_t>();
+    run(u, out, true);
+}
+
 void hogwild_fused_lse(at::Tensor& out, at::Tensor& rq, at::Tensor& lse, double scale, const at::Tensor& locations,
                        const at::Tensor& queries, const at::Tensor& fragment_lengths, const std::vector<at::Tensor>& key_fragments,
                        const std::vector<at::Tensor>& value_fragments, const at::Tensor& cosines, const at::Tensor& sines) {
@@ -386,6 +403,8 @@ TORCH_LIBRARY(libhogatt, m) {
           "Tensor fragment_lengths, Tensor[] key_fragments, Tensor[] value_fragments) -> ()", tags);
     m.def("hogwild_fused_lse(Tensor(a!) output, Tensor(b!) rq, Tensor(c!) lse, float scale, Tensor locations, Tensor queries, "
           "Tensor fragment_lengths, Tensor[] key_fragments, Tensor[] value_fragments, Tensor cosines, Tensor sines) -> ()", tags);
+    m.def("hogwild_fused_devlen(Tensor(a!) output, Tensor(b!) rq, float scale, Tensor locations, Tensor queries, "
+          "Tensor fragment_lengths, Tensor[] key_fragments, Tensor[] value_fragments, Tensor cosines, Tensor sines) -> ()", tags);
     // the paged operators, schemas of src/binding.cu:369-374
     m.def("hogwild_paged_sdpa(Tensor(a!) output, float scale, Tensor locations, Tensor queries, "
           "Tensor fragment_lengths, Tensor key_cache, Tensor value_cache, Tensor block_table) -> ()", tags);
@@ -401,6 +420,7 @@ TORCH_LIBRARY_IMPL(libhogatt, CUDA, m) {
     m.impl("hogwild_fused", hogwild_fused);
     m.impl("hogwild_sdpa_lse", hogwild_sdpa_lse);
     m.impl("hogwild_fused_lse", hogwild_fused_lse);
+    m.impl("hogwild_fused_devlen", hogwild_fused_devlen);
     m.impl("hogwild_paged_sdpa", hogwild_paged_sdpa);
     m.impl("copy_to_blocks", copy_to_blocks);
     m.impl("hogwild_varlen_paged_sdpa", hogwild_varlen_paged_sdpa);

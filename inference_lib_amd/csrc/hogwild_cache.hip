@@ -8,8 +8,11 @@
 //                           (:148-158), in one pass and in place.  With one source "worker" and a single
 //                           cos/sin row broadcast over its tokens this is also merge_caches (:251-257): re-rotate a
 //                           whole segment by a constant offset and append it to another.
+//   advance_lengths_kernel  len_dev[f] += add[f]: segment lengths kept in device memory, so that a decode step captured
+//                           as a graph can be replayed while the segments grow (the first two kernels and the
+//                           attention kernel then read the lengths from there).
 //
-// Both are tiny, latency-bound kernels; they exist so that a decode step needs no per-worker Python loop, no
+// All are tiny, latency-bound kernels; they exist so that a decode step needs no per-worker Python loop, no
 // torch.cat reallocation and no .contiguous() copy of the segments.
 
 #include <hip/hip_runtime.h>
@@ -37,7 +40,19 @@ __global__ __launch_bounds__(256) void build_inputs_kernel(const BuildInputsArgs
         const int tok = idx / per_tok;            // (f * W + w) * S + s
         const int s = tok % a.S;
         const int fw = tok / a.S;
-        const int pos = a.pos_end[fw] - a.S + s;
+        int pos_end;
+        if (a.len_dev == nullptr) {
+            pos_end = a.pos_end[fw];
+        } else {   // lengths in device memory: walk worker w's order from its end up to fragment f
+            const int f = fw / a.W, w = fw - f * a.W;
+            pos_end = 0;
+            for (int i = a.F - 1; i >= 0; --i) {
+                const int g = a.pos_end[w * a.F + i];
+                pos_end += a.len_dev[g];
+                if (g == f) break;
+            }
+        }
+        const int pos = pos_end - a.S + s;
         if (i == 0) a.locations[tok] = pos;
         if (half > 0) {
             // angle = float(position) * inv_freq, then cos / sin times the attention scaling, as the rotary
@@ -108,7 +123,11 @@ __global__ __launch_bounds__(256) void rope_append_kernel(const AppendArgs a) {
     const char* vsrc = reinterpret_cast<const char*>(a.v_src);
     char* kdst = reinterpret_cast<char*>(a.k_dst[w]);
     char* vdst = reinterpret_cast<char*>(a.v_dst[w]);
-    const int len = a.dst_len[w], cap = a.dst_cap[w];
+    const int cap = a.dst_cap[w];
+    // rows already in the segment: given, or (lengths in device memory) the segment's length after this append minus
+    // what is being appended; an append that would not fit is dropped rather than written outside the buffers
+    const int len = a.len_dev == nullptr ? a.dst_len[w] : a.len_dev[a.dst_len[w]] - n_new;
+    if (len < 0 || len + n_new > cap) return;
     for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
         const int c = (int)(idx % per_row);
         const long long row = idx / per_row;
@@ -172,6 +191,16 @@ hipError_t launch_build_inputs(const BuildInputsArgs& a, int round_dtype, hipStr
         case 2: hipLaunchKernelGGL((build_inputs_kernel<2>), dim3((unsigned)blocks), dim3(256), 0, stream, a); break;
         default: hipLaunchKernelGGL((build_inputs_kernel<0>), dim3((unsigned)blocks), dim3(256), 0, stream, a); break;
     }
+    return hipGetLastError();
+}
+
+__global__ __launch_bounds__(64) void advance_lengths_kernel(const AdvanceArgs a) {
+    const int f = threadIdx.x;
+    if (f < a.F) a.len_dev[f] += a.add[f];
+}
+
+hipError_t launch_advance_lengths(const AdvanceArgs& a, hipStream_t stream) {
+    hipLaunchKernelGGL(advance_lengths_kernel, dim3(1), dim3(64), 0, stream, a);
     return hipGetLastError();
 }
 

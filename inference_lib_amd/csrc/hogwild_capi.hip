@@ -49,6 +49,7 @@ int validate(const hw_problem* p, int fused) {
     if (p->out == nullptr || p->q == nullptr || p->locations == nullptr) return HW_ERR_NULL;
     if (p->k == nullptr || p->v == nullptr || p->len == nullptr) return HW_ERR_NULL;
     if (fused && p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
+    if (p->len_dev != nullptr && (!fused || p->RotE != p->E)) return HW_ERR_UNSUPPORTED;   // fused entry, full rotary width only
     long long rows = (long long)p->W * p->S * (p->Hq / p->Hkv);
     if (rows >= (1 << 20) || p->S >= (1 << 12) || p->Hq / p->Hkv >= (1 << 12)) return HW_ERR_SHAPE;
     if ((long long)p->Hkv * ((rows + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
@@ -200,12 +201,11 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     const size_t parts = (size_t)p->Hkv * plan.wgs_per_head;
     ka.h.part_o = reinterpret_cast<float*>(p->workspace);
     ka.h.part_ml = ka.h.part_o + parts * plan.rows * p->Ev;
+    ka.h.len_dev = p->len_dev;
     ka.h.F = p->F; ka.h.W = p->W; ka.h.Hq = p->Hq; ka.h.Hkv = p->Hkv; ka.h.S = p->S;
-    ka.h.RotE = prerotated ? 0 : p->RotE;
     ka.h.R = plan.rows;
     ka.h.nrg = plan.row_groups;
     ka.h.wgs_per_head = plan.wgs_per_head;
-    ka.h.tiles_per_head = plan.tiles_per_head;
     ka.h.nwg = plan.workgroups;
     ka.h.prerotated = prerotated ? 1 : 0;
     ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
@@ -424,11 +424,51 @@ int build_inputs_run(int32_t* locations, float* cosines, float* sines, const int
         a.inv_freq = inv_freq;
         a.scaling = scaling;
         a.F = nf; a.W = W; a.S = S; a.RotE = RotE;
+        a.len_dev = nullptr;
         std::memcpy(a.pos_end, pos_end + (size_t)f0 * W, sizeof(int) * (size_t)nf * W);
         hipError_t e = hw::launch_build_inputs(a, round_dtype, reinterpret_cast<hipStream_t>(stream));
         if (e != hipSuccess) return (int)e;
     }
     return HW_OK;
+}
+
+int build_inputs_dev_run(int32_t* locations, float* cosines, float* sines, const int32_t* len_dev, const int32_t* orders,
+                         const float* inv_freq, float scaling, int round_dtype, int F, int W, int S, int RotE, void* stream) {
+    if (F < 1 || F > HW_MAX_FRAGMENTS || W < 1 || S < 1 || RotE < 0 || (RotE & 1)) return HW_ERR_SHAPE;
+    if (round_dtype != HW_F32 && round_dtype != HW_F16 && round_dtype != HW_BF16) return HW_ERR_DTYPE;
+    if (locations == nullptr || len_dev == nullptr || orders == nullptr) return HW_ERR_NULL;
+    if (RotE > 0 && (cosines == nullptr || sines == nullptr || inv_freq == nullptr)) return HW_ERR_NULL;
+    if ((long long)F * W > hw::MAX_POS_ENTRIES) return HW_ERR_UNSUPPORTED;
+    if ((long long)F * W * S * (RotE > 0 ? RotE : 1) >= (1ll << 31)) return HW_ERR_SHAPE;
+    for (int w = 0; w < W; ++w) {      // every worker's order is a permutation of the fragments
+        unsigned seen = 0;
+        for (int i = 0; i < F; ++i) {
+            const int g = orders[(size_t)w * F + i];
+            if (g < 0 || g >= F || (seen >> g & 1u)) return HW_ERR_SHAPE;
+            seen |= 1u << g;
+        }
+    }
+    hw::BuildInputsArgs a;
+    a.locations = locations;
+    a.cosines = RotE > 0 ? cosines : nullptr;
+    a.sines = RotE > 0 ? sines : nullptr;
+    a.inv_freq = inv_freq;
+    a.scaling = scaling;
+    a.F = F; a.W = W; a.S = S; a.RotE = RotE;
+    a.len_dev = len_dev;
+    std::memcpy(a.pos_end, orders, sizeof(int) * (size_t)F * W);
+    return (int)hw::launch_build_inputs(a, round_dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+int advance_lengths_run(int32_t* len_dev, const int32_t* add, int F, void* stream) {
+    if (len_dev == nullptr || add == nullptr) return HW_ERR_NULL;
+    if (F < 1 || F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    hw::AdvanceArgs a;
+    std::memset(&a, 0, sizeof(a));
+    a.len_dev = len_dev;
+    a.F = F;
+    for (int f = 0; f < F; ++f) a.add[f] = add[f];
+    return (int)hw::launch_advance_lengths(a, reinterpret_cast<hipStream_t>(stream));
 }
 
 int rope_append_run(const hw_append* p, void* stream) {
@@ -442,7 +482,8 @@ int rope_append_run(const hw_append* p, void* stream) {
     bool any = false;
     for (int w = 0; w < p->W; ++w) {
         if (p->n_new[w] < 0 || p->n_new[w] > p->S || p->dst_len[w] < 0) return HW_ERR_SHAPE;
-        if ((long long)p->dst_len[w] + p->n_new[w] > p->dst_cap[w]) return HW_ERR_SHAPE;    // the segment is full
+        // (with the lengths in device memory dst_len is an index and the kernel itself drops what does not fit)
+        if (p->len_dev == nullptr && (long long)p->dst_len[w] + p->n_new[w] > p->dst_cap[w]) return HW_ERR_SHAPE;    // the segment is full
         if (p->n_new[w] > 0) {
             if (p->k_dst[w] == nullptr || p->v_dst[w] == nullptr) return HW_ERR_NULL;
             any = true;
@@ -471,6 +512,7 @@ int rope_append_run(const hw_append* p, void* stream) {
             a.dst_cap[w] = p->dst_cap[w0 + w];
             a.n_new[w] = p->n_new[w0 + w];
         }
+        a.len_dev = p->len_dev;
         hipError_t e = hw::launch_rope_append(a, p->dtype, p->mode == HW_ROPE_EAGER, p->cs_dtype != HW_F32, reinterpret_cast<hipStream_t>(stream));
         if (e != hipSuccess) return (int)e;
     }
@@ -585,6 +627,15 @@ int hw_build_inputs(int32_t* locations, float* cosines, float* sines, const int3
                     float attention_scaling, int round_dtype, int F, int W, int S, int RotE, void* stream) {
     return build_inputs_run(locations, cosines, sines, pos_end, inv_freq, attention_scaling, round_dtype, F, W, S, RotE, stream);
 }
+
+int hw_build_inputs_dev(int32_t* locations, float* cosines, float* sines, const int32_t* len_dev, const int32_t* orders,
+                        const float* inv_freq, float attention_scaling, int round_dtype, int F, int W, int S, int RotE,
+                        void* stream) {
+    return build_inputs_dev_run(locations, cosines, sines, len_dev, orders, inv_freq, attention_scaling, round_dtype, F, W, S, RotE,
+                                stream);
+}
+
+int hw_advance_lengths(int32_t* len_dev, const int32_t* add, int F, void* stream) { return advance_lengths_run(len_dev, add, F, stream); }
 
 int hw_rope_append(const hw_append* a, void* stream) { return rope_append_run(a, stream); }
 

@@ -486,8 +486,9 @@ struct DevHeader {
     HW_GLOBAL char* rq;
     HW_GLOBAL float* part_o;
     HW_GLOBAL float* part_ml;
-    int F, W, Hq, Hkv, S, RotE, R;
-    int nrg, wgs_per_head, tiles_per_head, nwg;
+    const HW_GLOBAL int* len_dev;
+    int F, W, Hq, Hkv, S, R;
+    int nrg, wgs_per_head, nwg;
     int prerotated;
     int xcd_remap;
     float sc;

@@ -34,8 +34,11 @@ struct alignas(64) KernelHeader {
     void* rq;
     float* part_o;      // [Hkv][wgs_per_head][R][Ev]  unnormalised partial outputs
     float* part_ml;     // [Hkv][wgs_per_head][R][2]   running max (base-2 units) and sum
-    int F, W, Hq, Hkv, S, RotE, R;
-    int nrg, wgs_per_head, tiles_per_head, nwg;
+    const int* len_dev; // [F] current fragment lengths in device memory, or null: the table's lengths are exact.
+                        // With it the table's lengths are the bounds the split was planned for and fragment f holds
+                        // min(bound, len_dev[f]) tokens, so a captured launch stays valid while segments grow.
+    int F, W, Hq, Hkv, S, R;
+    int nrg, wgs_per_head, nwg;
     int prerotated;
     int xcd_remap;
     float sc;           // scale * log2(e)
@@ -119,7 +122,12 @@ struct BuildInputsArgs {
     const float* inv_freq; // [RotE / 2]
     float scaling;
     int F, W, S, RotE;
-    int pos_end[MAX_POS_ENTRIES];   // [F][W]: position one past the newest token of worker w, as seen through fragment f
+    // pos_end[f][w]: position one past the newest token of worker w, as seen through fragment f.  Either given ...
+    int pos_end[MAX_POS_ENTRIES];
+    // ... or, with len_dev, formed in the kernel from the fragment lengths in device memory: the table then holds
+    // order[w][i] = the i-th fragment of worker w's order (W rows of F entries), and pos_end[f][w] is the sum of the
+    // lengths of f and of everything behind it in that order.
+    const int* len_dev;
 };
 
 struct AppendArgs {
@@ -131,12 +139,21 @@ struct AppendArgs {
     int W, Hkv, S, E, Ev, RotE;
     void* k_dst[MAX_APPEND_WORKERS];     // segment buffers [Hkv, cap, E] / [Hkv, cap, Ev]
     void* v_dst[MAX_APPEND_WORKERS];
-    int dst_len[MAX_APPEND_WORKERS];     // rows already in the segment
+    int dst_len[MAX_APPEND_WORKERS];     // rows already in the segment; with len_dev: index into len_dev, whose entry
+                                         // is the segment's length AFTER this append (rows already there = entry - n_new)
     int dst_cap[MAX_APPEND_WORKERS];
     int n_new[MAX_APPEND_WORKERS];       // the last n_new of the S source tokens are appended
+    const int* len_dev;                  // segment lengths in device memory, or null
 };
 
 hipError_t launch_build_inputs(const BuildInputsArgs& a, int round_dtype, hipStream_t stream);
 hipError_t launch_rope_append(const AppendArgs& a, int dtype, bool eager, bool cs16, hipStream_t stream);
+// len_dev[f] += add[f] for f < F (F <= MAXF): the first node of a captured decode step
+struct AdvanceArgs {
+    int* len_dev;
+    int F;
+    int add[MAXF];
+};
+hipError_t launch_advance_lengths(const AdvanceArgs& a, hipStream_t stream);
 
 }  // namespace hw

@@ -59,7 +59,9 @@ namespace hw {
 // MINW = waves per SIMD the register budget is sized for: 2 (<= 256 VGPRs) when one 16-row block is live,
 // 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the tile registers too large.
 // PF = tiles a wave keeps in flight.  PRE = queries arrive rotated (hogwild_sdpa), else fused rotation.
-template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE>
+// DEVLEN = the current fragment lengths come from device memory (header.len_dev); the lengths in the table are then
+// the bounds the split was planned for, and a captured launch stays valid while the segments grow up to them.
+template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE, bool DEVLEN = false>
 __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     constexpr int ROWS = RB * 16;
@@ -94,7 +96,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
     const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
     const FragTable::LenCap my_lc = args.frag.lc[fl];
-    const int my_len = my_lc.len, my_cap = my_lc.cap;
+    int my_len = my_lc.len;
+    const int my_cap = my_lc.cap;
     const int my_tb = args.frag.tile_begin[fl];
     const int my_te = args.frag.tile_begin[fl + 1];
     int my_wt[MAX_SPLITS / 64], my_wt1[MAX_SPLITS / 64];
@@ -123,6 +126,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     st.fresh = true;
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");   // the header is usable from here on
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
+    if constexpr (DEVLEN) my_len = min(my_len, a.len_dev[fl < a.F ? fl : 0]);
 
     // consecutive logical ids stay on one XCD (hardware deals workgroups round-robin over the 8 XCDs)
     int bid = blockIdx.x;
@@ -170,6 +174,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
         fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW);
         lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
         lt1 = s1 - fb;
+        if constexpr (DEVLEN) lt1 = min(lt1, (L + TILE - 1) / TILE);   // the fragment may be shorter than planned (or empty)
         opens_fragment = s0 == fb;
         // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first K/V tile; the
         // rotation then waits only for the former while the tile stays in flight
@@ -404,25 +409,31 @@ __global__ __launch_bounds__(256) void stream_copy_kernel(u32x4* dst, const u32x
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
-template <class DT, int E, int EV, bool PRE>
+template <class DT, int E, int EV, bool PRE, bool DEVLEN>
 static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t stream) {
     constexpr bool half = Elem<DT>::size == 2;
     if (rb == 1)
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
                            stream, ka);
     else
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, half ? HW_MINW2 : 1, half ? HW_PF2 : 1, PRE>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, half ? HW_MINW2 : 1, half ? HW_PF2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg),
+                           dim3(NTHREADS), 0, stream, ka);
     return hipGetLastError();
 }
 
 template <class DT>
 static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, hipStream_t stream) {
     if (ka.h.prerotated) {
-        if (E == 128) return launch_attention_rb<DT, 128, 128, true>(ka, rb, stream);
-        return launch_attention_rb<DT, 64, 64, true>(ka, rb, stream);
+        if (ka.h.len_dev != nullptr) return hipErrorInvalidValue;   // device-resident lengths exist for the fused entry only
+        if (E == 128) return launch_attention_rb<DT, 128, 128, true, false>(ka, rb, stream);
+        return launch_attention_rb<DT, 64, 64, true, false>(ka, rb, stream);
     }
-    if (E == 128) return launch_attention_rb<DT, 128, 128, false>(ka, rb, stream);
-    return launch_attention_rb<DT, 64, 64, false>(ka, rb, stream);
+    if (ka.h.len_dev != nullptr) {
+        if (E == 128) return launch_attention_rb<DT, 128, 128, false, true>(ka, rb, stream);
+        return launch_attention_rb<DT, 64, 64, false, true>(ka, rb, stream);
+    }
+    if (E == 128) return launch_attention_rb<DT, 128, 128, false, false>(ka, rb, stream);
+    return launch_attention_rb<DT, 64, 64, false, false>(ka, rb, stream);
 }
 
 hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream) {

@@ -64,7 +64,8 @@ class AttentionModule(nn.Module):
         # queries are rotated per fragment inside the operator (attention.py:326-339)
         rq = cache.get_queries_buffer(query_states, layer_idx=self.layer_idx)
         attn = hogwild_fused(query_states, cs.loc, cs.keys, cs.values, self.scaling, cs.frags, cs.cos, cs.sin,
-                             rotated_queries=rq, out=cache.get_att_buffer(rq, layer_idx=self.layer_idx))
+                             rotated_queries=rq, out=cache.get_att_buffer(rq, layer_idx=self.layer_idx),
+                             device_lengths=cache.device_lengths)
         attn = attn.transpose(1, 2).reshape(*input_shape, -1).contiguous()
         return self.o_proj(attn), None
 

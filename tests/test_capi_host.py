@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
     for name in declared:
         assert hasattr(L.lib, name), name
-    assert L.lib.hw_version() == 2
+    assert L.lib.hw_version() == 3
 
 
 def test_struct_layout_matches_header():
@@ -128,6 +128,24 @@ def test_plan_invariants(lens, kw):
             assert all(a < b for a, b in zip(wb, wb[1:])) or tiles == 0          # every workgroup owns at least one tile
             assert pl.workgroups == n * kw["Hkv"] * pl.row_groups
             assert pl.workspace_bytes >= kw["Hkv"] * n * pl.rows * (kw["Ev"] + 2) * 4
+
+
+def test_device_length_entry_points_validate_on_the_host():
+    L = _lib()
+    # device-resident lengths exist for the fused entry with full rotary width only
+    assert L.lib.hw_validate(C.byref(_problem(L, len_dev=0x1000)), 1) == 0
+    assert L.lib.hw_validate(C.byref(_problem(L, len_dev=0x1000)), 0) == -4
+    assert L.lib.hw_validate(C.byref(_problem(L, len_dev=0x1000, RotE=64)), 1) == -4
+    orders = (C.c_int32 * 6)(0, 1, 2, 0, 2, 1)
+    bi = lambda o, F=3, W=2, **kw: L.lib.hw_build_inputs_dev(kw.get("loc", 0x1000), 0x1000, 0x1000, kw.get("ld", 0x1000), o, 0x1000,
+                                                            1.0, kw.get("rd", 0), F, W, 1, kw.get("rot", 64), None)
+    assert bi(None) == -1 and bi(orders, loc=None) == -1 and bi(orders, ld=None) == -1
+    assert bi(orders, rd=7) == -2 and bi(orders, rot=63) == -3 and bi(orders, F=33) == -3
+    assert bi((C.c_int32 * 6)(0, 1, 1, 0, 2, 1)) == -3            # a fragment twice in one worker's order
+    assert bi((C.c_int32 * 6)(0, 1, 3, 0, 2, 1)) == -3            # not a fragment
+    add = (C.c_int32 * 3)(0, 1, 1)
+    assert L.lib.hw_advance_lengths(None, add, 3, None) == -1 and L.lib.hw_advance_lengths(0x1000, None, 3, None) == -1
+    assert L.lib.hw_advance_lengths(0x1000, add, 0, None) == -5 and L.lib.hw_advance_lengths(0x1000, add, 33, None) == -5
 
 
 def test_plan_spreads_tiny_fragments():

@@ -290,3 +290,84 @@ def test_segment_grows_when_full():
     torch.cuda.synchronize()
     assert seg.get_seq_length(1) == 10 and seg.get_seq_length(0) == 0 and seg.k[1].size(1) >= 10 and seg.k[0].size(1) == 3
     assert torch.equal(seg.key_cache[1], torch.cat(parts_k, dim=2)) and torch.equal(seg.value_cache[1], torch.cat(parts_v, dim=2))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+def test_decode_steps_replayed_from_one_graph_with_device_lengths(dtype):
+    """The same three-worker, two-layer decode loop twice: cache A with host-side lengths, stepped eagerly (the path the
+    test above checks against the oracles), and cache B with the lengths in device memory, whose step is captured in a
+    HIP graph once and replayed while its segments grow.  Every step must give the same attention output (the split is
+    planned for different lengths, so to tolerance, not bit for bit), and at the end the segments must hold the same
+    rows bit for bit."""
+    from inference_lib_amd import attention, cache
+    tdt = TDT[dtype]
+    g = torch.Generator().manual_seed(29)
+    layers, W, Hq, Hkv, D, S = 2, 3, 8, 2, 128, 1
+    f = torch.from_numpy(inv_freq(D)).to(DEV)
+    scale = D ** -0.5
+    P = [40, 7, 0, 19]                                                     # prompt and what the workers have written so far
+
+    def make():
+        segs = [cache.SegmentCache(layers, Hkv, D, 8, dtype=tdt, device=DEV) for _ in range(1 + W)]
+        gg = torch.Generator().manual_seed(3)
+        for i, n in enumerate(P):
+            for layer in range(layers):
+                if n:
+                    segs[i].update(torch.randn((1, Hkv, n, D), generator=gg).to(tdt).to(DEV), torch.randn((1, Hkv, n, D), generator=gg).to(tdt).to(DEV), layer)
+        orders = [[0] + [1 + o for o in range(W) if o != w] + [1 + w] for w in range(W)]
+        return segs, cache.HogwildCache([[segs[i] for i in o] for o in orders], inv_freq=f)
+
+    segs_a, hc_a = make()
+    segs_b, hc_b = make()
+    hc_b.use_device_lengths(headroom=16, new_tokens=S)
+    qbuf = torch.zeros((layers, W, Hq, S, D), dtype=tdt, device=DEV)
+    kbuf = torch.zeros((layers, W, S, Hkv, D), dtype=tdt, device=DEV)
+    vbuf = torch.zeros((layers, W, S, Hkv, D), dtype=tdt, device=DEV)
+    out_a = torch.zeros((layers, W, Hq, S, D), dtype=tdt, device=DEV)
+    out_b = torch.zeros((layers, W, Hq, S, D), dtype=tdt, device=DEV)
+    ids = torch.zeros((W, S), dtype=torch.int64, device=DEV)
+
+    def step(hc, outs):
+        pos = hc.get_input_kwargs(ids)["position_ids"]
+        ang = pos.to(torch.float32)[..., None] * f
+        emb = torch.cat([ang, ang], dim=-1)
+        cos_k, sin_k = emb.cos().to(tdt), emb.sin().to(tdt)
+        for layer in range(layers):
+            cs = hc.update_fused(kbuf[layer].transpose(1, 2), vbuf[layer].transpose(1, 2), cos_k, sin_k, layer)
+            rq = hc.get_queries_buffer(qbuf[layer], layer)
+            o = attention.hogwild_fused(qbuf[layer], cs.loc, cs.keys, cs.values, scale, cs.frags, cs.cos, cs.sin, rotated_queries=rq,
+                                        out=hc.get_att_buffer(rq, layer), device_lengths=hc.device_lengths)
+            outs[layer].copy_(o)
+
+    def new_inputs():
+        qbuf.copy_(torch.randn(qbuf.shape, generator=g).to(tdt))
+        kbuf.copy_(torch.randn(kbuf.shape, generator=g).to(tdt))
+        vbuf.copy_(torch.randn(vbuf.shape, generator=g).to(tdt))
+
+    tol = TOL[dtype]
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        new_inputs()
+        step(hc_a, out_a)                       # step 0 eagerly on both (warms the capture stream up as well)
+        step(hc_b, out_b)
+        torch.cuda.synchronize()
+        assert (out_a.float() - out_b.float()).abs().max().item() <= tol
+        with torch.cuda.graph(graph, stream=stream):
+            step(hc_b, out_b)
+        for it in range(1, 7):
+            new_inputs()
+            step(hc_a, out_a)
+            torch.cuda.synchronize()
+            print(f"replay {it}: device lengths {hc_b._dev['len_dev'].tolist()}", flush=True)
+            graph.replay()
+            torch.cuda.synchronize()
+            err = (out_a.float() - out_b.float()).abs().max().item()
+            assert torch.isfinite(out_b.float()).all() and err <= tol, (it, err)
+            (out_b.float().sum() + 1).item()    # eager work between the replays
+    hc_b.use_host_lengths()
+    for sa, sb in zip(segs_a, segs_b):
+        assert sa.lengths == sb.lengths == [sa.lengths[0]] * layers
+        for layer in range(layers):
+            assert torch.equal(sa.key_cache[layer], sb.key_cache[layer]) and torch.equal(sa.value_cache[layer], sb.value_cache[layer])
+    assert [s.get_seq_length() for s in segs_b] == [P[0]] + [p + 7 for p in P[1:]]

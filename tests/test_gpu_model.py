@@ -125,3 +125,48 @@ def test_left_masked_workers():
         want_b = plain(torch.cat([p_ids[0], a_ids, b_ids])[None]).logits[0, -1].float()
     assert (got[0, -1] - want_a).abs().max().item() <= tol
     assert (got[1, -1] - want_b).abs().max().item() <= tol
+
+
+def test_decode_steps_replayed_from_one_graph():
+    """The whole decode step of the swapped model (embedding, rotary embedding, both decoder layers with key rotation +
+    append + fused attention, head) captured in a HIP graph once, with the segment lengths in device memory, and replayed
+    while the worker's segment grows; every replay must give the plain model's logits at that position."""
+    from inference_lib_amd.cache import HogwildCache
+    from inference_lib_amd.model import decode_step
+    dtype, tol = torch.float32, 5e-5
+    cfg, plain = tiny_model(2, dtype, seed=4)
+    hog = swapped_copy(plain)
+    T, N = 21, 9
+    g = torch.Generator().manual_seed(13)
+    ids = torch.randint(0, cfg.vocab_size, (1, T + N), generator=g).to(DEV)
+    with torch.no_grad():
+        want = plain(ids).logits.float()
+    prompt, seg = segment(cfg, 32, dtype), segment(cfg, 4, dtype)
+    decode_step(hog, HogwildCache([[prompt]], hog), ids[:, :T])
+    cache = HogwildCache([[prompt, seg]], hog)
+    cache.use_device_lengths(headroom=16, new_tokens=1)
+    tok = torch.zeros((1, 1), dtype=ids.dtype, device=DEV)
+    logits = torch.zeros((1, 1, cfg.vocab_size), dtype=dtype, device=DEV)
+
+    def step():
+        logits.copy_(decode_step(hog, cache, tok))
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        tok.copy_(ids[:, T: T + 1])
+        step()                                   # first token eagerly
+        torch.cuda.synchronize()
+        assert (logits.float() - want[:, T: T + 1]).abs().max().item() <= tol
+        with torch.cuda.graph(graph, stream=stream):
+            step()
+        for i in range(1, N):
+            tok.copy_(ids[:, T + i: T + i + 1])
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            err = (logits.float() - want[:, T + i: T + i + 1]).abs().max().item()
+            print(f"replay {i}: max err {err:.3e}", flush=True)
+            assert err <= tol
+    cache.use_host_lengths()
+    assert seg.get_seq_length() == N and prompt.get_seq_length() == T
