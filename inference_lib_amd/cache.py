@@ -118,11 +118,12 @@ class HogwildCache:
         self._dev = None        # state of the device-resident-lengths mode, see use_device_lengths
 
     # ---- lengths in device memory: decode steps that can be captured once and replayed ------------------------------
-    def use_device_lengths(self, headroom: int, new_tokens: int = 1) -> None:
+    def use_device_lengths(self, headroom: int, new_tokens: int = 1, n_new: Optional[Sequence[int]] = None) -> None:
         """From now on the segment lengths live in a device tensor that every step advances on the device, so a decode
         step (update_fused + hogwild_fused for every layer) can be captured in a HIP graph once and replayed while the
-        segments grow: nothing about a step depends on host numbers any more.  Every worker appends `new_tokens` tokens
-        per step (no left masking in this mode).  The attention split is planned for lengths up to `headroom` tokens
+        segments grow: nothing about a step depends on host numbers any more.  Every step brings `new_tokens` tokens per
+        worker, of which worker w appends the last n_new[w] (left masking with the same mask in every step; default: all
+        of them).  The attention split is planned for lengths up to `headroom` tokens
         beyond the present ones, and the buffers are grown to hold them now, so a capture is good for
         headroom // new_tokens steps; call this again to re-plan.  The host-side lengths are not touched by the steps:
         sync_lengths() reads them back.  No counterpart in the reference, whose segments are re-allocated on every
@@ -132,9 +133,14 @@ class HogwildCache:
         for seg in segments:
             if len(set(seg.lengths)) != 1:
                 raise ValueError("all layers of a segment must hold the same number of tokens (call between decode steps)")
+        if len({id(seg) for seg in self.write_to}) != len(self.write_to):
+            raise ValueError("with device-resident lengths every worker needs a segment of its own to write to")
+        n_new = [int(new_tokens)] * len(self.write_to) if n_new is None else [int(x) for x in n_new]
+        if len(n_new) != len(self.write_to) or any(x < 0 or x > int(new_tokens) for x in n_new):
+            raise ValueError("n_new: one number per worker, between 0 and new_tokens")
         add = [0] * len(segments)
-        for seg in self.write_to:
-            add[index[id(seg)]] += int(new_tokens)
+        for seg, n in zip(self.write_to, n_new):
+            add[index[id(seg)]] += n
         bound = [seg.get_seq_length() + (int(headroom) if add[f] else 0) for f, seg in enumerate(segments)]
         for f, seg in enumerate(segments):
             for layer in range(len(seg.k)):
@@ -143,6 +149,7 @@ class HogwildCache:
         self._dev = {
             "segments": segments, "orders": [[index[id(cs)] for cs in order] for order in self.cache_structure],
             "write_index": [index[id(seg)] for seg in self.write_to], "add": add, "S": int(new_tokens), "bound": bound,
+            "n_new": n_new, "n_new_dev": torch.tensor(n_new, dtype=torch.int64, device=dev),
             "len_dev": torch.tensor([seg.get_seq_length() for seg in segments], dtype=torch.int32, device=dev),
             "write_index_dev": torch.tensor([index[id(seg)] for seg in self.write_to], dtype=torch.int64, device=dev),
             "tables": None,
@@ -180,7 +187,7 @@ class HogwildCache:
             self.frags = d["len_dev"]
         segs = self.write_to
         _lib.rope_append(key_states, value_states, [s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs], d["write_index"],
-                         cosines=cos, sines=sin, mode=mode, len_dev=d["len_dev"])
+                         cosines=cos, sines=sin, n_new=d["n_new"], mode=mode, len_dev=d["len_dev"])
         # the fragments as the operator sees them: views up to the planned bounds, current lengths in `frags`
         keys = [seg.k[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
         vals = [seg.v[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
@@ -196,12 +203,19 @@ class HogwildCache:
         S = key_states.size(2)
         n_new = [S] * W if mask is None else [int(x) for x in torch.sum(mask, dim=1).tolist()]   # left masking, :149-155
         segs = self.write_to
+        # workers that write to the same segment append one behind the other, in worker order (the reference's loop, :148-158)
+        end: Dict[int, int] = {}
+        dst = []
         for s, n in zip(segs, n_new):
-            s.reserve(layer_idx, n)
+            start = end.get(id(s), s.lengths[layer_idx])
+            dst.append(start)
+            end[id(s)] = start + n
+        for s in segs:
+            s.reserve(layer_idx, end[id(s)] - s.lengths[layer_idx])
         _lib.rope_append(key_states, value_states, [s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs],
-                         [s.lengths[layer_idx] for s in segs], cosines=cosines, sines=sines, n_new=n_new, mode=mode)
-        for s, n in zip(segs, n_new):
-            s.lengths[layer_idx] += n
+                         dst, cosines=cosines, sines=sines, n_new=n_new, mode=mode)
+        for s in segs:
+            s.lengths[layer_idx] = end[id(s)]
 
     def _structure(self, key_states, layer_idx) -> CacheStructure:
         W, S = key_states.size(0), key_states.size(2)
@@ -229,8 +243,6 @@ class HogwildCache:
         """key_states [W, Hkv, S, D] already rotated (the reference rotates them before the call, attention.py:315)."""
         mask = (cache_kwargs or {}).get("mask", None)
         if self._dev is not None:
-            if mask is not None:
-                raise ValueError("left masking is not available with device-resident lengths")
             return self._update_dev(key_states, value_states, None, None, layer_idx, _lib.HW_ROPE_EAGER)
         self._append(key_states, value_states, layer_idx, mask, None, None, _lib.HW_ROPE_EAGER)
         return self._structure(key_states, layer_idx)
@@ -239,9 +251,7 @@ class HogwildCache:
                      mask: Optional[torch.Tensor] = None, mode: int = _lib.HW_ROPE_EAGER) -> CacheStructure:
         """The same with un-rotated keys and the model's position embeddings cos/sin [W, S, RotE] of the new tokens:
         rotation (attention.py:313-315) and append (:148-158) in one launch."""
-        if self._dev is not None:
-            if mask is not None:
-                raise ValueError("left masking is not available with device-resident lengths")
+        if self._dev is not None:      # (a mask, if given, must be the one n_new was derived from; it is not read here)
             return self._update_dev(key_states, value_states, cos, sin, layer_idx, mode)
         self._append(key_states, value_states, layer_idx, mask, cos, sin, mode)
         return self._structure(key_states, layer_idx)
@@ -264,11 +274,10 @@ class HogwildCache:
         assert input_ids.shape[0] == nw, (input_ids.shape, nw)
         S = input_ids.shape[1]
         if self._dev is not None:      # positions from the lengths in device memory (before this step's append)
-            if attention_mask is not None:
-                raise ValueError("left masking is not available with device-resident lengths")
-            start = self._dev["len_dev"].index_select(0, self._dev["write_index_dev"]).to(torch.int64)
-            pos_ids = start[:, None] + torch.arange(S, dtype=torch.int64, device=input_ids.device)[None, :]
-            return {"input_ids": input_ids, "attention_mask": None, "past_key_values": self, "use_cache": True, "position_ids": pos_ids}
+            ends = self._dev["len_dev"].index_select(0, self._dev["write_index_dev"]).to(torch.int64) + self._dev["n_new_dev"]
+            pos_ids = ends[:, None] - S + torch.arange(S, dtype=torch.int64, device=input_ids.device)[None, :]
+            return {"input_ids": input_ids, "attention_mask": attention_mask, "past_key_values": self, "use_cache": True,
+                    "position_ids": pos_ids}
         new = [S] * nw if attention_mask is None else [int(x) for x in torch.sum(attention_mask, dim=1).tolist()]
         ends = torch.tensor([self.cache_structure[w][-1].get_seq_length() + new[w] for w in range(nw)], dtype=torch.int64, device=input_ids.device)
         pos_ids = ends[:, None] - S + torch.arange(S, dtype=torch.int64, device=input_ids.device)[None, :]

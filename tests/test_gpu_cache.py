@@ -371,3 +371,26 @@ def test_decode_steps_replayed_from_one_graph_with_device_lengths(dtype):
         for layer in range(layers):
             assert torch.equal(sa.key_cache[layer], sb.key_cache[layer]) and torch.equal(sa.value_cache[layer], sb.value_cache[layer])
     assert [s.get_seq_length() for s in segs_b] == [P[0]] + [p + 7 for p in P[1:]]
+
+
+def test_workers_that_share_a_write_segment_append_in_worker_order():
+    """Two workers writing to one segment: worker 0's tokens first, then worker 1's (the reference updates the caches
+    in a loop over the workers, python/hogwild/attention.py:148-158)."""
+    from inference_lib_amd import cache
+    Hkv, D = 2, 64
+    shared = cache.SegmentCache(1, Hkv, D, 4, dtype=torch.float16, device=DEV)
+    other = cache.SegmentCache(1, Hkv, D, 4, dtype=torch.float16, device=DEV)
+    hc = cache.HogwildCache([[other, shared], [other, shared], [shared, other]], inv_freq=torch.from_numpy(inv_freq(D)).to(DEV),
+                            write_to=[shared, shared, other])
+    g = torch.Generator().manual_seed(2)
+    k = torch.randn((3, Hkv, 2, D), generator=g).half().to(DEV)
+    v = torch.randn((3, Hkv, 2, D), generator=g).half().to(DEV)
+    mask = torch.tensor([[1, 1], [0, 1], [1, 1]], device=DEV)
+    hc.update(k, v, 0, {"mask": mask})
+    torch.cuda.synchronize()
+    assert shared.get_seq_length() == 3 and other.get_seq_length() == 2
+    assert torch.equal(shared.key_cache[0][0], torch.cat([k[0], k[1, :, 1:]], dim=1))
+    assert torch.equal(shared.value_cache[0][0], torch.cat([v[0], v[1, :, 1:]], dim=1))
+    assert torch.equal(other.key_cache[0][0], k[2])
+    with pytest.raises(ValueError):
+        hc.use_device_lengths(8)

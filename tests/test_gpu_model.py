@@ -125,6 +125,20 @@ def test_left_masked_workers():
         want_b = plain(torch.cat([p_ids[0], a_ids, b_ids])[None]).logits[0, -1].float()
     assert (got[0, -1] - want_a).abs().max().item() <= tol
     assert (got[1, -1] - want_b).abs().max().item() <= tol
+    # the same kind of step (three tokens for worker 0, one for worker 1) with the lengths in device memory
+    a2 = torch.randint(0, cfg.vocab_size, (3,), generator=g).to(DEV)
+    b2 = torch.randint(0, cfg.vocab_size, (1,), generator=g).to(DEV)
+    cache.use_device_lengths(headroom=8, new_tokens=3, n_new=[3, 1])
+    ids2 = torch.stack([a2, torch.cat([torch.zeros(2, dtype=a2.dtype, device=DEV), b2])])
+    print("masked step, device-resident lengths", flush=True)
+    got2 = decode_step(hog, cache, ids2, mask).float()
+    cache.use_host_lengths()
+    assert sa.get_seq_length() == 6 and sb.get_seq_length() == 2
+    with torch.no_grad():
+        want_a2 = plain(torch.cat([p_ids[0], b_ids, b2, a_ids, a2])[None]).logits[0, -1].float()
+        want_b2 = plain(torch.cat([p_ids[0], a_ids, a2, b_ids, b2])[None]).logits[0, -1].float()
+    assert (got2[0, -1] - want_a2).abs().max().item() <= tol
+    assert (got2[1, -1] - want_b2).abs().max().item() <= tol
 
 
 def test_decode_steps_replayed_from_one_graph():
