@@ -69,3 +69,37 @@ def test_paged_random_shapes(seed):
     else:
         c = build_paged(dtype, F, W, Hkv * GQ, Hkv, D, bs, mb, seq_lens=seq, S=S, **kw)
     check_paged(c, splits=int(rng.choice([0, 0, 1, 5])))
+
+
+@pytest.mark.parametrize("seed", range(18))
+def test_fused_random_shapes_with_device_lengths(oracle, seed):
+    """The same sweep through the device-resident-lengths path: every fragment sits in a buffer that is longer than
+    its current length (the planned bound, 0..70 tokens more, sometimes with nothing written yet), the rows beyond the
+    length are NaN, and the lengths reach the kernel through device memory only."""
+    from inference_lib_amd import _lib
+    c, splits = random_case(seed)
+    rng = np.random.default_rng(500 + seed)
+    dev = torch.device("cuda:0")
+    cd = c.to(dev)
+    keys, values = [], []
+    for k, v in zip(cd.keys, cd.values):
+        extra = int(rng.choice([0, 1, 31, 32, 33, 70]))
+        pad_k = torch.full((k.size(0), extra, k.size(2)), float("nan"), dtype=k.dtype, device=dev)
+        pad_v = torch.full((v.size(0), extra, v.size(2)), float("nan"), dtype=v.dtype, device=dev)
+        keys.append(torch.cat([k, pad_k], dim=1).contiguous())
+        values.append(torch.cat([v, pad_v], dim=1).contiguous())
+    len_dev = torch.tensor(c.lens, dtype=torch.int32, device=dev)
+    W, Hq, S, E = cd.q.shape
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=dev)
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=dev)
+    rq = torch.full((c.F, W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=dev)
+    print(f"seed {seed}: {c.dtype} E={c.E} W={c.W} S={c.S} Hq={c.Hq} Hkv={c.Hkv} lens={c.lens} bounds={[k.size(1) for k in keys]} "
+          f"splits={splits}", flush=True)
+    _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=values, scale=c.scale, out=out, cosines=cd.cos, sines=cd.sin,
+                 rq=rq, lse=lse, splits=splits, len_dev=len_dev).run()
+    torch.cuda.synchronize()
+    want_o, want_l, want_rq = oracle_fused(oracle, c)
+    tol = TOL[c.dtype]
+    assert_close("out", out, want_o, tol)
+    assert_close("lse", lse, want_l, tol)
+    assert_close("rq", rq, want_rq, 1e-5 if c.dtype == "f32" else 3.2e-2)
