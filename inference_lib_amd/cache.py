@@ -163,8 +163,21 @@ class HogwildCache:
         """Device-resident lengths -> host-side lengths of every segment and layer (synchronises with the device)."""
         if self._dev is None:
             return
-        for seg, n in zip(self._dev["segments"], self._dev["len_dev"].tolist()):
+        lens = self._dev["len_dev"].tolist()
+        over = [f for f, (n, b) in enumerate(zip(lens, self._dev["bound"])) if n > b]
+        if over:
+            raise RuntimeError(f"segments {over} grew beyond the lengths the steps were planned for ({lens} vs {self._dev['bound']}): "
+                               "the captured step was replayed more often than headroom // new_tokens; the tokens beyond the bounds "
+                               "were not attended to")
+        for seg, n in zip(self._dev["segments"], lens):
             seg.lengths = [int(n)] * len(seg.lengths)
+
+    def device_steps_left(self) -> int:
+        """How many more steps the current plan covers (reads the lengths back: synchronises with the device)."""
+        if self._dev is None:
+            raise ValueError("not in the device-resident-lengths mode")
+        lens = self._dev["len_dev"].tolist()
+        return min(((b - n) // a for n, b, a in zip(lens, self._dev["bound"], self._dev["add"]) if a > 0), default=0)
 
     def use_host_lengths(self) -> None:
         """Leave the device-resident-lengths mode (after reading the lengths back)."""

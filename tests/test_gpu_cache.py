@@ -365,6 +365,7 @@ def test_decode_steps_replayed_from_one_graph_with_device_lengths(dtype):
             err = (out_a.float() - out_b.float()).abs().max().item()
             assert torch.isfinite(out_b.float()).all() and err <= tol, (it, err)
             (out_b.float().sum() + 1).item()    # eager work between the replays
+    assert hc_b.device_steps_left() == 16 - 7
     hc_b.use_host_lengths()
     for sa, sb in zip(segs_a, segs_b):
         assert sa.lengths == sb.lengths == [sa.lengths[0]] * layers
@@ -394,3 +395,17 @@ def test_workers_that_share_a_write_segment_append_in_worker_order():
     assert torch.equal(other.key_cache[0][0], k[2])
     with pytest.raises(ValueError):
         hc.use_device_lengths(8)
+
+
+def test_replaying_beyond_the_planned_lengths_is_reported():
+    from inference_lib_amd import _lib, cache
+    Hkv, D = 2, 64
+    seg = cache.SegmentCache(1, Hkv, D, 64, dtype=torch.float16, device=DEV)
+    hc = cache.HogwildCache([[seg]], inv_freq=torch.from_numpy(inv_freq(D)).to(DEV))
+    hc.use_device_lengths(headroom=2)
+    assert hc.device_steps_left() == 2
+    for _ in range(3):
+        _lib.advance_lengths(hc._dev["len_dev"], hc._dev["add"])
+    assert hc.device_steps_left() < 0
+    with pytest.raises(RuntimeError):
+        hc.sync_lengths()
