@@ -1,6 +1,7 @@
 /*
  * A caller of the C ABI written in plain C: no torch, no C++.  One fused decode step (hw_fused_attention) and one
- * paged step (hw_copy_to_blocks + hw_paged_sdpa) on inputs whose answer has a closed form:
+ * paged step (hw_copy_to_blocks + hw_paged_sdpa) on inputs whose answer has a closed form (the fused step also with the
+ * fragment lengths in device memory):
  * with q = 0 every visible key gets the same weight, so out = mean of the visible V rows and lse = ln(count).
  * V[f][h][l][e] = (l % 7) + f + 0.25 * h + e / 64, exactly representable in fp32.
  * Exit code 0 and a line "c_abi ok" on success.
@@ -102,6 +103,43 @@ int main(void) {
         }
     printf("fused: worst deviation from the closed form %.3e\n", worst);
     if (!(worst < 1e-4)) return 4;
+
+    /* the same launch with the current lengths in device memory: the fragment buffers are the planned bounds, the
+       kernel sees min(bound, len_dev[f]) tokens; hw_advance_lengths moves the lengths on the device */
+    {
+        int cur[F] = {48, 33, 0};
+        const int add[F] = {2, 0, 0};                               /* -> 50, 33, 0 */
+        void* dlen = to_device(cur, sizeof(cur));
+        if (!dlen) return 2;
+        CHECK_HW(hw_advance_lengths((int32_t*)dlen, add, F, stream));
+        p.len_dev = (const int32_t*)dlen;
+        CHECK_HW(hw_fused_attention(&p, stream));
+        CHECK_HIP(hipStreamSynchronize(stream));
+        p.len_dev = NULL;
+        CHECK_HIP(hipMemcpy(out, dout, sizeof(out), hipMemcpyDeviceToHost));
+        CHECK_HIP(hipMemcpy(lse, dlse, sizeof(lse), hipMemcpyDeviceToHost));
+        const int now[F] = {50, 33, 0};
+        worst = 0.0;
+        for (int w = 0; w < W; ++w)
+            for (int h = 0; h < HQ; ++h) {
+                int hk = h / (HQ / HKV), count = 0;
+                double mean[D];
+                memset(mean, 0, sizeof(mean));
+                for (int f = 0; f < F; ++f) {
+                    int vis = loc[f][w][0] + 1 < now[f] ? loc[f][w][0] + 1 : now[f];
+                    for (int l = 0; l < vis; ++l, ++count)
+                        for (int e = 0; e < D; ++e) mean[e] += vval(f, hk, l, e);
+                }
+                for (int e = 0; e < D; ++e) {
+                    double err = fabs(out[w][h][0][e] - mean[e] / count);
+                    if (err > worst) worst = err;
+                }
+                double el = fabs(lse[w][h][0] - log((double)count));
+                if (el > worst) worst = el;
+            }
+        printf("fused, lengths in device memory: worst deviation from the closed form %.3e\n", worst);
+        if (!(worst < 1e-4)) return 7;
+    }
 
     /* an unsupported head dimension is an error, not a silent no-op */
     p.E = p.Ev = 96;
