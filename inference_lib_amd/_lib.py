@@ -643,6 +643,73 @@ def rope_append(key_states: torch.Tensor, value_states: torch.Tensor, k_dst: Seq
         check(lib.hw_rope_append(C.byref(a), C.c_void_p(stream)), "hw_rope_append")
 
 
+class AppendPlan:
+    """hw_rope_append with everything that stays the same from step to step prepared once: destination buffers,
+    capacities, tokens per worker, and the segment lengths in device memory.  run() fills in the new states and their
+    rotary tables and launches; it checks only what can change between calls."""
+
+    def __init__(self, k_dst: Sequence[torch.Tensor], v_dst: Sequence[torch.Tensor], seg_index: Sequence[int], n_new: Sequence[int],
+                 len_dev: torch.Tensor, mode: int = HW_ROPE_EAGER):
+        W = len(k_dst)
+        if len(v_dst) != W or len(seg_index) != W or len(n_new) != W:
+            raise ValueError("one destination segment, length index and token count per worker")
+        kd0 = k_dst[0]
+        for kd, vd in zip(k_dst, v_dst):
+            if kd.dim() != 3 or vd.dim() != 3 or kd.shape[:2] != vd.shape[:2] or not kd.is_contiguous() or not vd.is_contiguous() \
+                    or kd.size(0) != kd0.size(0) or kd.size(2) != kd0.size(2) or vd.size(2) != v_dst[0].size(2) \
+                    or kd.dtype != kd0.dtype or vd.dtype != kd0.dtype or kd.device != kd0.device:
+                raise ValueError("segment buffers must be contiguous [Hkv, cap, E|Ev] of one dtype on one device")
+        if len_dev.dtype != torch.int32 or len_dev.dim() != 1 or not len_dev.is_contiguous() or len_dev.device != kd0.device:
+            raise ValueError("len_dev must be a contiguous int32 vector on the device of the segments")
+        if any(int(x) < 0 or int(x) >= len_dev.numel() for x in seg_index):
+            raise ValueError("seg_index holds indices into len_dev")
+        self.W, self.Hkv, self.E, self.Ev = W, kd0.size(0), kd0.size(2), v_dst[0].size(2)
+        self.dtype, self.device = kd0.dtype, kd0.device
+        self._keep = (list(k_dst), list(v_dst), len_dev)
+        self._kp = (C.c_void_p * W)(*[t.data_ptr() for t in k_dst])
+        self._vp = (C.c_void_p * W)(*[t.data_ptr() for t in v_dst])
+        self._ln = (C.c_int32 * W)(*[int(x) for x in seg_index])
+        self._cp = (C.c_int32 * W)(*[t.size(1) for t in k_dst])
+        self._nn = (C.c_int32 * W)(*[int(x) for x in n_new])
+        a = HwAppend()
+        a.dtype = _DTYPE_CODE[self.dtype]
+        a.mode = int(mode)
+        a.W, a.Hkv, a.E, a.Ev = W, self.Hkv, self.E, self.Ev
+        a.k_dst, a.v_dst = C.cast(self._kp, C.POINTER(C.c_void_p)), C.cast(self._vp, C.POINTER(C.c_void_p))
+        a.dst_len, a.dst_cap, a.n_new = (C.cast(self._ln, C.POINTER(C.c_int32)), C.cast(self._cp, C.POINTER(C.c_int32)),
+                                         C.cast(self._nn, C.POINTER(C.c_int32)))
+        a.len_dev = len_dev.data_ptr()
+        self.a = a
+
+    def run(self, key_states: torch.Tensor, value_states: torch.Tensor, cosines: Optional[torch.Tensor] = None,
+            sines: Optional[torch.Tensor] = None) -> None:
+        a = self.a
+        W, Hkv, S, E = key_states.shape
+        if (W, Hkv, E) != (self.W, self.Hkv, self.E) or tuple(value_states.shape) != (W, Hkv, S, self.Ev) \
+                or key_states.dtype != self.dtype or value_states.dtype != self.dtype or key_states.device != self.device:
+            raise ValueError("new states do not match the prepared append")
+        if (E > 1 and key_states.stride(3) != 1) or (self.Ev > 1 and value_states.stride(3) != 1):
+            key_states, value_states = key_states.contiguous(), value_states.contiguous()
+        a.S = S
+        a.key_states, a.value_states = key_states.data_ptr(), value_states.data_ptr()
+        a.ks_w, a.ks_h, a.ks_s = key_states.stride(0), key_states.stride(1), key_states.stride(2)
+        a.vs_w, a.vs_h, a.vs_s = value_states.stride(0), value_states.stride(1), value_states.stride(2)
+        if cosines is None:
+            a.RotE, a.cs_dtype, a.cosines, a.sines = 0, HW_F32, None, None
+        else:
+            if sines is None or cosines.shape != sines.shape or cosines.dim() != 3 or cosines.size(0) != W or cosines.size(1) not in (1, S) \
+                    or cosines.dtype != sines.dtype or cosines.dtype not in (torch.float32, self.dtype):
+                raise ValueError("cosines / sines must be [W, S, RotE] or [W, 1, RotE], float32 or in the dtype of the keys")
+            cosines, sines = cosines.contiguous(), sines.contiguous()
+            a.RotE = cosines.size(2)
+            a.cs_dtype = _DTYPE_CODE[cosines.dtype]
+            a.cosines, a.sines = cosines.data_ptr(), sines.data_ptr()
+            a.cs_w = cosines.stride(0)
+            a.cs_s = 0 if cosines.size(1) == 1 else cosines.stride(1)
+        stream = torch.cuda.current_stream(self.device).cuda_stream
+        check(lib.hw_rope_append(C.byref(a), C.c_void_p(stream)), "hw_rope_append")
+
+
 def rope(q: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     F, W, Hq, S, E = out.shape
     if tuple(q.shape) != (W, Hq, S, E) or q.dtype != out.dtype:

@@ -152,7 +152,7 @@ class HogwildCache:
             "n_new": n_new, "n_new_dev": torch.tensor(n_new, dtype=torch.int64, device=dev),
             "len_dev": torch.tensor([seg.get_seq_length() for seg in segments], dtype=torch.int32, device=dev),
             "write_index_dev": torch.tensor([index[id(seg)] for seg in self.write_to], dtype=torch.int64, device=dev),
-            "tables": None,
+            "tables": None, "views": {}, "appends": {},
         }
 
     @property
@@ -198,13 +198,21 @@ class HogwildCache:
             self.locations, self.cosines, self.sines = d["tables"]
             self.segments = d["segments"]
             self.frags = d["len_dev"]
-        segs = self.write_to
-        _lib.rope_append(key_states, value_states, [s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs], d["write_index"],
-                         cosines=cos, sines=sin, n_new=d["n_new"], mode=mode, len_dev=d["len_dev"])
-        # the fragments as the operator sees them: views up to the planned bounds, current lengths in `frags`
-        keys = [seg.k[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
-        vals = [seg.v[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])]
-        return CacheStructure(keys=keys, values=vals, cos=self.cosines, sin=self.sines, loc=self.locations, frags=self.frags)
+        plan = d["appends"].get((layer_idx, mode))
+        if plan is None:        # destinations, capacities and token counts stay the same from step to step
+            segs = self.write_to
+            plan = _lib.AppendPlan([s.k[layer_idx] for s in segs], [s.v[layer_idx] for s in segs], d["write_index"], d["n_new"],
+                                   d["len_dev"], mode)
+            d["appends"][(layer_idx, mode)] = plan
+        plan.run(key_states, value_states, cos, sin)
+        # the fragments as the operator sees them: views up to the planned bounds (the same in every step, so they are
+        # made once per layer), current lengths in `frags`
+        views = d["views"].get(layer_idx)
+        if views is None:
+            views = ([seg.k[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])],
+                     [seg.v[layer_idx][:, :b, :].unsqueeze(0) for seg, b in zip(d["segments"], d["bound"])])
+            d["views"][layer_idx] = views
+        return CacheStructure(keys=views[0], values=views[1], cos=self.cosines, sin=self.sines, loc=self.locations, frags=self.frags)
 
     def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
         return self.cache_structure[0][-1].get_seq_length()        # attention.py:133-135
