@@ -50,9 +50,12 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
     ap.add_argument("--ring-mb", type=int, default=640)
-    ap.add_argument("--workload", choices=["fragments", "paged", "varlen"], default="fragments",
+    ap.add_argument("--workload", choices=["fragments", "paged", "varlen", "stack"], default="fragments",
                     help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape; "
-                         "varlen = hogwild_varlen_paged_sdpa on the same cache with 1 / 8 / 32 / 64 query tokens per sequence")
+                         "varlen = hogwild_varlen_paged_sdpa on the same cache with 1 / 8 / 32 / 64 query tokens per sequence; "
+                         "stack = the attention part of a 64-layer decode step through HogwildCache (append + attention + merge per "
+                         "layer), eagerly and as one HIP graph")
+    ap.add_argument("--layers", type=int, default=64, help="stack workload: decoder layers")
     ap.add_argument("--seq-len", type=int, default=12528, help="paged workload: tokens per sequence")
     ap.add_argument("--block-size", type=int, default=16, help="paged workload: tokens per cache block")
     return ap.parse_args()
@@ -95,6 +98,9 @@ def main():
 
     if args.workload in ("paged", "varlen"):
         bench_paged(args, dev)
+        return
+    if args.workload == "stack":
+        bench_stack(args, dev)
         return
 
     case = cases.baseline_case(args.case)
@@ -461,6 +467,93 @@ def bench_paged(args, dev):
         result["cpu_baseline"] = {"value": round(kv_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                                   "us_per_step": round(med * 1e6, 1),
                                   "sample": f"{len(ts)} full steps of the same workload (median), numpy fp32 restatement of the paged kernel"}
+    print(json.dumps(result, ensure_ascii=False))
+
+
+def bench_stack(args, dev):
+    """The attention part of one decode step of a whole model at the headline shape: per layer the new keys are rotated
+    and appended to every worker's segment (hw_rope_append), then attention + merge (hogwild_fused); at layer 0 the
+    step's locations and rotary tables are built.  Every layer has its own KV buffers (prompt of 4096 tokens, four
+    worker segments of 2048), so a step streams layers x 51 MB.  Three ways of driving it: eagerly from Python with
+    host-side lengths, eagerly with the lengths in device memory, and the latter captured once as a HIP graph and
+    replayed.  `value` is the graph replay."""
+    import torch
+    from inference_lib_amd import attention, cache
+    L, W, Hq, Hkv, D, S = args.layers, 4, 40, 8, 128, 1
+    tdt = torch.bfloat16
+    seg_lens = [4096, 2048, 2048, 2048, 2048]
+    inv = (1e6 ** (-torch.arange(0, D, 2, dtype=torch.float32) / D)).to(dev)
+    orders = [[0] + [1 + o for o in range(W) if o != w] + [1 + w] for w in range(W)]
+
+    def make():
+        segs = [cache.SegmentCache(L, Hkv, D, n + 160, dtype=tdt, device=dev) for n in seg_lens]
+        for sg, n in zip(segs, seg_lens):
+            sg.lengths = [n] * L
+            for layer in range(L):
+                sg.k[layer].normal_()
+                sg.v[layer].normal_()
+        return cache.HogwildCache([[segs[i] for i in o] for o in orders], inv_freq=inv)
+
+    q = torch.randn((W, Hq, S, D), device=dev).to(tdt)
+    kn = torch.randn((W, S, Hkv, D), device=dev).to(tdt).transpose(1, 2)
+    vn = torch.randn((W, S, Hkv, D), device=dev).to(tdt).transpose(1, 2)
+    ids = torch.zeros((W, S), dtype=torch.int64, device=dev)
+
+    def step(hc):
+        pos = hc.get_input_kwargs(ids)["position_ids"]
+        ang = pos.to(torch.float32)[..., None] * inv
+        emb = torch.cat([ang, ang], dim=-1)
+        ck, sk = emb.cos().to(tdt), emb.sin().to(tdt)
+        for layer in range(L):
+            cs = hc.update_fused(kn, vn, ck, sk, layer)
+            rq = hc.get_queries_buffer(q, layer)
+            attention.hogwild_fused(q, cs.loc, cs.keys, cs.values, D ** -0.5, cs.frags, cs.cos, cs.sin, rotated_queries=rq,
+                                    out=hc.get_att_buffer(rq, layer), device_lengths=hc.device_lengths)
+
+    K, Wm = min(args.steps, 40), min(args.warmup, 5)
+
+    def timed(fn, n):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e6
+
+    hc_a = make()
+    for _ in range(Wm):
+        step(hc_a)
+    eager_host_us = timed(lambda: step(hc_a), K)
+    del hc_a
+    hc_b = make()
+    hc_b.use_device_lengths(headroom=2 * (K + Wm) + 8)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        for _ in range(Wm):
+            step(hc_b)
+        eager_dev_us = timed(lambda: step(hc_b), K)
+        with torch.cuda.graph(graph, stream=stream):
+            step(hc_b)
+        for _ in range(Wm):
+            graph.replay()
+        graph_us = timed(graph.replay, K)
+    left = hc_b.device_steps_left()
+    assert left >= 0, "replayed beyond the planned lengths"
+    kv_bytes = L * sum(seg_lens) * Hkv * 2 * D * 2
+    value = kv_bytes / (graph_us * 1e-6) / 1e9
+    result = {
+        "metric": METRIC + f", attention part of a {L}-layer decode step (key rotation + append, attention, merge per layer)",
+        "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": Wm, "ms_per_step": round(graph_us / 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"decode stack: {L} layers, W=4 S=1 Hq=40 Hkv=8 D=128 bf16, segments {seg_lens} per layer, "
+                               "lengths in device memory, one HIP graph per step", "kv_bytes_per_step": kv_bytes},
+        "roofline": {"bound": "hbm", "achieved": round(value, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(value / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "whole step (3 kernels per layer)",
+                     "timing": "wall clock around K graph replays"},
+        "extra": {"graph_us_per_layer": round(graph_us / L, 2), "eager_device_lengths_us_per_layer": round(eager_dev_us / L, 2),
+                  "eager_host_lengths_us_per_layer": round(eager_host_us / L, 2), "planned_steps_left": left},
+    }
     print(json.dumps(result, ensure_ascii=False))
 
 
