@@ -41,7 +41,7 @@ extern "C" {
 #endif
 
 #define HW_ABI_VERSION 3
-#define HW_MAX_FRAGMENTS 32
+#define HW_MAX_FRAGMENTS 64
 #define HW_MAX_SPLITS 256      /* workgroups per kv head */
 
 typedef enum hw_status {

@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
 
-HW_MAX_FRAGMENTS = 32
+HW_MAX_FRAGMENTS = 64
 HW_MAX_SPLITS = 256
 HW_F32, HW_F16, HW_BF16 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_BF16}

@@ -441,11 +441,11 @@ int build_inputs_dev_run(int32_t* locations, float* cosines, float* sines, const
     if ((long long)F * W > hw::MAX_POS_ENTRIES) return HW_ERR_UNSUPPORTED;
     if ((long long)F * W * S * (RotE > 0 ? RotE : 1) >= (1ll << 31)) return HW_ERR_SHAPE;
     for (int w = 0; w < W; ++w) {      // every worker's order is a permutation of the fragments
-        unsigned seen = 0;
+        unsigned long long seen = 0;
         for (int i = 0; i < F; ++i) {
             const int g = orders[(size_t)w * F + i];
-            if (g < 0 || g >= F || (seen >> g & 1u)) return HW_ERR_SHAPE;
-            seen |= 1u << g;
+            if (g < 0 || g >= F || (seen >> g & 1ull)) return HW_ERR_SHAPE;
+            seen |= 1ull << g;
         }
     }
     hw::BuildInputsArgs a;

@@ -6,7 +6,7 @@
 
 namespace hw {
 
-constexpr int MAXF = 32;       // fragments per launch (table travels in the kernel arguments)
+constexpr int MAXF = 64;       // fragments per launch (table travels in the kernel arguments)
 constexpr int TILE = 32;       // tokens per wave step
 constexpr int NWAVES = 4;      // waves per workgroup
 constexpr int NTHREADS = NWAVES * 64;

@@ -81,7 +81,7 @@ def test_validation_happens_on_the_host():
     assert v(_problem(L, scale=-1.0)) == -3
     assert v(_problem(L, E=96, Ev=96, RotE=96)) == -4       # valid but not instantiated: a hard error, never silent
     assert v(_problem(L, Ev=64)) == -4
-    assert v(_problem(L, F=33)) == -5
+    assert v(_problem(L, F=65)) == -5
     assert v(_problem(L, F=0)) == -5
     assert v(_problem(L, out=None)) == -1
     assert v(_problem(L, cosines=None)) == -1
@@ -140,12 +140,12 @@ def test_device_length_entry_points_validate_on_the_host():
     bi = lambda o, F=3, W=2, **kw: L.lib.hw_build_inputs_dev(kw.get("loc", 0x1000), 0x1000, 0x1000, kw.get("ld", 0x1000), o, 0x1000,
                                                             1.0, kw.get("rd", 0), F, W, 1, kw.get("rot", 64), None)
     assert bi(None) == -1 and bi(orders, loc=None) == -1 and bi(orders, ld=None) == -1
-    assert bi(orders, rd=7) == -2 and bi(orders, rot=63) == -3 and bi(orders, F=33) == -3
+    assert bi(orders, rd=7) == -2 and bi(orders, rot=63) == -3 and bi(orders, F=65) == -3
     assert bi((C.c_int32 * 6)(0, 1, 1, 0, 2, 1)) == -3            # a fragment twice in one worker's order
     assert bi((C.c_int32 * 6)(0, 1, 3, 0, 2, 1)) == -3            # not a fragment
     add = (C.c_int32 * 3)(0, 1, 1)
     assert L.lib.hw_advance_lengths(None, add, 3, None) == -1 and L.lib.hw_advance_lengths(0x1000, None, 3, None) == -1
-    assert L.lib.hw_advance_lengths(0x1000, add, 0, None) == -5 and L.lib.hw_advance_lengths(0x1000, add, 33, None) == -5
+    assert L.lib.hw_advance_lengths(0x1000, add, 0, None) == -5 and L.lib.hw_advance_lengths(0x1000, add, 65, None) == -5
 
 
 def test_plan_spreads_tiny_fragments():
@@ -214,7 +214,7 @@ def test_paged_validation_happens_on_the_host():
     assert v(_paged(L)) == 0
     assert L.lib.hw_paged_validate(None) == -1
     assert v(_paged(L, dtype=5)) == -2
-    assert v(_paged(L, F=0)) == -5 and v(_paged(L, F=33)) == -5
+    assert v(_paged(L, F=0)) == -5 and v(_paged(L, F=65)) == -5
     assert v(_paged(L, Hq=41)) == -3
     assert v(_paged(L, scale=0.0)) == -3 and v(_paged(L, scale=float("nan"))) == -3
     assert v(_paged(L, block_size=0)) == -3 and v(_paged(L, block_size=4096)) == -3

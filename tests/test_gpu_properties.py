@@ -103,11 +103,11 @@ def test_rows_that_see_nothing_and_empty_fragments(oracle):
 
 def test_fragment_limit(oracle):
     from inference_lib_amd import _lib, cases
-    lens = [40] + [3 + (i % 5) for i in range(31)]
-    W = 31
+    lens = [40] + [3 + (i % 5) for i in range(63)]
+    W = 63
     c = cases.build_case("f32max", "bf16", W, 1, 2 * W // W * 2, 2, 64, 1e4, lens, [[0, 1 + w] for w in range(W)],
                          torch.Generator().manual_seed(3))
-    assert c.F == 32
+    assert c.F == 64
     out, lse, _ = run_fused(c.to(_dev()))
     o_ref, l_ref, _ = oracle_fused(oracle, c)
     assert_close("out", out, o_ref, TOL["bf16"])
