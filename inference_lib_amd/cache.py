@@ -215,6 +215,9 @@ class HogwildCache:
         return CacheStructure(keys=views[0], values=views[1], cos=self.cosines, sin=self.sines, loc=self.locations, frags=self.frags)
 
     def get_seq_length(self, layer_idx: Optional[int] = 0) -> int:
+        if self._dev is not None:      # the host-side lengths are stale in this mode: read the device's (synchronises)
+            f = [id(cs) for cs in self._dev["segments"]].index(id(self.cache_structure[0][-1]))
+            return int(self._dev["len_dev"][f].item())
         return self.cache_structure[0][-1].get_seq_length()        # attention.py:133-135
 
     # ---- the append ------------------------------------------------------------------------------------------------

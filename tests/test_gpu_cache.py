@@ -366,6 +366,7 @@ def test_decode_steps_replayed_from_one_graph_with_device_lengths(dtype):
             assert torch.isfinite(out_b.float()).all() and err <= tol, (it, err)
             (out_b.float().sum() + 1).item()    # eager work between the replays
     assert hc_b.device_steps_left() == 16 - 7
+    assert hc_b.get_seq_length() == hc_a.get_seq_length()        # read from the device in this mode
     hc_b.use_host_lengths()
     for sa, sb in zip(segs_a, segs_b):
         assert sa.lengths == sb.lengths == [sa.lengths[0]] * layers
