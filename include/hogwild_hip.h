@@ -54,7 +54,8 @@ typedef enum hw_status {
     HW_ERR_FRAGMENTS = -5,     /* F < 1 or F > HW_MAX_FRAGMENTS */
     HW_ERR_WORKSPACE = -6,     /* workspace NULL or smaller than hw_workspace_bytes() */
     HW_ERR_ALIGN = -7,         /* a device pointer is not 16-byte aligned */
-    HW_ERR_NO_DEVICE = -8      /* no usable HIP device */
+    HW_ERR_NO_DEVICE = -8,     /* no usable HIP device */
+    HW_ERR_STATIC_SCRATCH = -9 /* hw_fused_attention_static: the problem needs more than HW_STATIC_SCRATCH_BYTES */
 } hw_status;
 
 typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
@@ -140,6 +141,19 @@ int hw_workspace_bytes(const hw_problem* p, size_t* bytes);
 
 /* Rotate q per fragment in registers and attend; replaces hogwild_fused. */
 int hw_fused_attention(const hw_problem* p, void* stream);
+
+/*
+ * hw_fused_attention for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same inputs, outputs and kernels as
+ * hw_fused_attention, except that p->workspace / p->workspace_bytes are ignored: the split-K partials go to a
+ * device array that is part of the library image (HW_STATIC_SCRATCH_BYTES per GPU, resident until the process ends).
+ * The call allocates and frees nothing.  A problem whose hw_workspace_bytes() exceeds HW_STATIC_SCRATCH_BYTES is
+ * refused with HW_ERR_STATIC_SCRATCH before anything is queued.  All calls on one GPU share that GPU's array: calls
+ * that overlap in time on one GPU (different streams, or graphs replayed concurrently) race on the partials and
+ * must be serialised by the caller.  Nothing in the array has to survive between calls or start at zero.
+ */
+#define HW_STATIC_SCRATCH_BYTES (8u << 20)
+int hw_fused_attention_static(const hw_problem* p, void* stream);
 
 /* The two kernels of hw_fused_attention separately.  HW_STAGE_ATTENTION leaves the split-K partials of this
    device's KV in the workspace (per kv head and workgroup: unnormalised output rows, running max in base-2 units

@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
 
 HW_MAX_FRAGMENTS = 64
 HW_MAX_SPLITS = 256
+HW_STATIC_SCRATCH_BYTES = 8 << 20
 HW_F32, HW_F16, HW_BF16 = 0, 1, 2
 _DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_BF16}
 
@@ -27,7 +28,7 @@ EXPORTS = [
     "hw_stream_read", "hw_stream_copy",
     "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
     "hw_paged_sdpa_stages", "hw_copy_to_blocks", "hw_build_inputs", "hw_rope_append",
-    "hw_build_inputs_dev", "hw_advance_lengths",
+    "hw_build_inputs_dev", "hw_advance_lengths", "hw_fused_attention_static",
 ]
 
 
@@ -131,6 +132,7 @@ def _load() -> C.CDLL:
     lib.hw_workspace_bytes.argtypes = [C.POINTER(HwProblem), C.POINTER(C.c_size_t)]
     lib.hw_fused_attention.argtypes = [C.POINTER(HwProblem), C.c_void_p]
     lib.hw_sdpa.argtypes = [C.POINTER(HwProblem), C.c_void_p]
+    lib.hw_fused_attention_static.argtypes = [C.POINTER(HwProblem), C.c_void_p]
     lib.hw_fused_attention_stages.argtypes = [C.POINTER(HwProblem), C.c_void_p, C.c_int]
     lib.hw_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                             C.c_int, C.c_int, C.c_int, C.c_void_p]
@@ -323,6 +325,15 @@ class Problem:
                 return
             fn = lib.hw_sdpa if self.prerotated else lib.hw_fused_attention
             check(fn(C.byref(self.p), C.c_void_p(stream)), fn.__name__)
+
+
+    def run_static(self) -> None:
+        """hw_fused_attention_static: the same step with the partials in the library's own device array; allocates nothing."""
+        if self.prerotated:
+            raise ValueError("the static-scratch entry exists for the fused operator only")
+        with torch.cuda.device(self.device):
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+            check(lib.hw_fused_attention_static(C.byref(self.p), C.c_void_p(stream)), "hw_fused_attention_static")
 
 
 def plan(lens: Sequence[int], *, W: int, S: int, Hq: int, Hkv: int, Ev: int, num_cus: int, splits: int = 0,

@@ -32,6 +32,28 @@ int device_cus(int* cus) {
     return HW_OK;
 }
 
+// Scratch of hw_fused_attention_static: the split-K partials (and, for rotary widths other than the head dimension,
+// the rotated queries) of callers that cannot allocate.  One copy per GPU, held until the process ends.  On the host
+// the array's name is only a handle: the device address comes from hipGetSymbolAddress, once per device.
+__attribute__((used)) static __device__ __align__(256) unsigned char scratch[HW_STATIC_SCRATCH_BYTES];
+std::atomic<void*> g_scratch[kMaxDevices];   // device address of `scratch` on each device; null = not asked yet
+
+int static_scratch(void** ptr) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return HW_ERR_NO_DEVICE;
+    void* p = g_scratch[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (p == nullptr) return HW_ERR_NO_DEVICE;
+        g_scratch[dev].store(p, std::memory_order_release);
+    }
+    *ptr = p;
+    return HW_OK;
+}
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 size_t elem_size(int dtype) { return dtype == HW_F32 ? 4 : 2; }
@@ -536,6 +558,7 @@ const char* hw_status_string(int status) {
         case HW_ERR_WORKSPACE: return "workspace missing, misaligned or too small";
         case HW_ERR_ALIGN: return "device pointer not 16-byte aligned";
         case HW_ERR_NO_DEVICE: return "no usable HIP device";
+        case HW_ERR_STATIC_SCRATCH: return "problem needs more scratch than HW_STATIC_SCRATCH_BYTES (use hw_fused_attention with a caller workspace)";
         default: break;
     }
     if (status > 0) return hipGetErrorString(static_cast<hipError_t>(status));
@@ -569,6 +592,25 @@ int hw_workspace_bytes(const hw_problem* p, size_t* bytes) {
 int hw_fused_attention(const hw_problem* p, void* stream) { return run(p, stream, 1); }
 
 int hw_sdpa(const hw_problem* p, void* stream) { return run(p, stream, 0); }
+
+int hw_fused_attention_static(const hw_problem* p, void* stream) {
+    int st = validate(p, 1);
+    if (st != HW_OK) return st;
+    int cus = 0;
+    st = device_cus(&cus);
+    if (st != HW_OK) return st;
+    hw_plan plan;
+    st = make_plan(p, cus, &plan);
+    if (st != HW_OK) return st;
+    if (plan.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES) return HW_ERR_STATIC_SCRATCH;
+    void* ptr = nullptr;
+    st = static_scratch(&ptr);
+    if (st != HW_OK) return st;
+    hw_problem q = *p;
+    q.workspace = ptr;
+    q.workspace_bytes = (size_t)HW_STATIC_SCRATCH_BYTES;
+    return run(&q, stream, 1);
+}
 
 int hw_fused_attention_stages(const hw_problem* p, void* stream, int stages) {
     if ((stages & (HW_STAGE_ATTENTION | HW_STAGE_MERGE)) == 0 || (stages & ~(HW_STAGE_ATTENTION | HW_STAGE_MERGE)) != 0) return HW_ERR_SHAPE;

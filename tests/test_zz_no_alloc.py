@@ -1,0 +1,90 @@
+"""hw_fused_attention_static (the entry point that allocates nothing: split-K partials in a device array that is part
+of the library image) against hw_fused_attention on the same inputs, through the C ABI.  Same kernels, same split
+plan, so the results must be bit-identical.  Two calls in a row, the second with a smaller input, because every call
+on a GPU shares that GPU's array and finds the previous call's contents in it."""
+import pytest
+import torch
+
+from helpers import TOL, assert_close, oracle_fused
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")
+
+
+def _both(case):
+    """(out, lse, rq) of the workspace entry point and of the static-scratch entry point."""
+    from inference_lib_amd import _lib
+    cd = case.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    res = []
+    for static in (False, True):
+        out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+        rq = torch.full((case.F, W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out,
+                          cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse)
+        if static:
+            pr.run_static()
+        else:
+            pr.run()
+        torch.cuda.synchronize()
+        res.append((out, lse, rq))
+    return res
+
+
+def test_static_scratch_matches_workspace_entry(oracle):
+    from inference_lib_amd import cases
+    big = cases.baseline_case(3)                      # headline shape: 256 workgroups, 2.7 MB of partials
+    small = cases.small_case(dtype="bf16", W=2, S=1, Hq=8, Hkv=2, E=128, lens=(100, 37, 65), seed=11)
+    part = cases.small_case(dtype="f16", W=3, S=2, Hq=6, Hkv=2, E=64, lens=(70, 33, 1, 64), seed=5)   # prompt + 3 segments
+    for c in (big, small, part, big):                 # larger, smaller, other dtype / head dim, larger again
+        print(f"case {c.name} lens={c.lens}", flush=True)
+        (o0, l0, r0), (o1, l1, r1) = _both(c)
+        assert torch.equal(o0, o1), "out differs between the two entry points"
+        assert torch.equal(l0, l1), "lse differs between the two entry points"
+        assert torch.equal(r0.view(torch.int16), r1.view(torch.int16)), "rotated queries differ"
+        o_ref, l_ref, _ = oracle_fused(oracle, c)
+        assert_close("out", o1, o_ref, TOL[c.dtype])
+        assert_close("lse", l1, l_ref, TOL[c.dtype])
+
+
+def test_static_scratch_partial_rotary_uses_the_array_for_the_rotated_queries(oracle):
+    """Rotary width != head dim: the standalone rotation writes the rotated queries into the scratch as well."""
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype="bf16", W=2, S=1, Hq=8, Hkv=2, E=128, lens=(90, 40, 17), seed=3, rot_dim=64)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    outs = []
+    for static in (False, True):
+        out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out,
+                          cosines=cd.cos, sines=cd.sin)
+        pr.run_static() if static else pr.run()
+        torch.cuda.synchronize()
+        outs.append(out)
+    assert torch.equal(outs[0], outs[1])
+    o_ref, _, _ = oracle_fused(oracle, c)
+    assert_close("out", outs[1], o_ref, TOL[c.dtype])
+
+
+def test_static_scratch_refuses_what_does_not_fit():
+    """A problem whose partials exceed the array is refused on the host, before anything is queued."""
+    from inference_lib_amd import _lib
+    dev = _dev()
+    W, Hq, Hkv, S, E = 64, 64, 8, 4, 128               # 2048 rows per kv head
+    L = 4096
+    q = torch.zeros((W, Hq, S, E), dtype=torch.bfloat16, device=dev)
+    k = torch.zeros((Hkv, L, E), dtype=torch.bfloat16, device=dev)
+    loc = torch.full((1, W, S), L - 1, dtype=torch.int32, device=dev)
+    cs = torch.zeros((1, W, S, E), dtype=torch.float32, device=dev)
+    out = torch.empty_like(q)
+    pr = _lib.Problem(q=q, locations=loc, keys=[k], values=[k], scale=0.1, out=out, cosines=cs, sines=cs)
+    assert pr.workspace_bytes() > _lib.HW_STATIC_SCRATCH_BYTES
+    with pytest.raises(_lib.HogwildError) as ei:
+        pr.run_static()
+    assert ei.value.status == -9
+    assert "HW_STATIC_SCRATCH_BYTES" in str(ei.value)
