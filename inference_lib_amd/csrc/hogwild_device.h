@@ -146,12 +146,15 @@ struct TileRegs {
 struct FragView {
     __amdgpu_buffer_rsrc_t k;
     unsigned long long vbase;   // start of the kv head's V rows
+    unsigned long long idle;    // where the V loads of a tile that does not exist go: a line every workgroup keeps hot
     int L;
 };
 constexpr unsigned OOB_OFFSET = 0xFFFF0000u;   // beyond any fragment (lengths are validated on the host)
 
-__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow) {
+__device__ __forceinline__ FragView make_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow,
+                                              unsigned long long idle) {
     FragView fv;
+    fv.idle = idle;
     fv.k = __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(kptr + (unsigned long long)hkv * cap * krow), 0, L * krow, 0x00020000);
     fv.vbase = vptr + (unsigned long long)hkv * cap * vrow;
     fv.L = L;
@@ -193,12 +196,13 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
     for (int i = 0; i < G::KL; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, HW_KV_AUX);
     // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load.  Rows beyond the fragment are
-    // redirected to its last row (their probabilities are zero); a tile that does not exist re-reads the first bytes
-    // of the fragment with every lane (one cache line per instruction).
+    // redirected to its last row (their probabilities are zero); a tile that does not exist reads one cached line
+    // (fv.idle) with every lane: loads return in order, so what such a load costs is its own latency behind the last
+    // real tile, and that must be a cache hit, not a trip to memory.
 #pragma unroll
     for (int idx = 0; idx < 8; ++idx) {
         const int row = min(t0 + q * 4 + (idx >> 2) * 16 + (idx & 3), fv.L - 1);
-        const unsigned long long addr = fv.vbase + (real ? (unsigned long long)(unsigned)row * G::VROW + n * (G::VLD * 4) : 0ull);
+        const unsigned long long addr = real ? fv.vbase + (unsigned long long)(unsigned)row * G::VROW + n * (G::VLD * 4) : fv.idle;
 #pragma unroll
         for (int hh = 0; hh < G::NVL; ++hh) {
             if constexpr (G::VLD == 4) {
@@ -413,65 +417,80 @@ template <> struct Chunk<F16> {
 
 
 // What each wave of a workgroup hands over at the end (row stride padded so that rows land in different banks).
+// The four waves' references and sums of one row lie next to each other: one 16-byte read fetches all of them.
 template <int ROWS, int EV>
 struct Exchange {
     float o[NWAVES][ROWS][EV + 4];
-    float m[NWAVES][ROWS];
-    float l[NWAVES][ROWS];
+    float m[ROWS][NWAVES];
+    float l[ROWS][NWAVES];
 };
 
 // Epilogue shared by the attention kernels: every wave hands over its raw accumulators, running max and sum
 // through LDS (one barrier); then all threads combine them with the weights 2^(m_wave - m_max) and store the
 // workgroup's partial coalesced: `nrows` rows starting at partial row index `part` (EV floats per row in part_o,
-// a (max, sum) pair per row in part_ml).  `ex` may alias a K staging slot: the leading barrier makes sure every
-// wave is done with it.
-template <class DT, int EV, int RB>
+// a (max, sum) pair per row in part_ml).  ALIASED: `ex` shares its memory with a K staging slot, so nobody may
+// write it before every wave is done with its tiles; otherwise each wave hands over as soon as it is done, while
+// the slower waves of the workgroup still compute, and only the combine follows the barrier.  Rows beyond `nrows`
+// (MFMA padding) are neither written nor read.
+template <class DT, int EV, int RB, bool ALIASED>
 __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Exchange<RB * 16, EV>& ex, int wv, int n, int q, int tid,
                                                HW_GLOBAL float* part_o, HW_GLOBAL float* part_ml, size_t part, int nrows) {
     constexpr int NOC = EV / 16;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) st.l[rb] = quarter_sum(st.l[rb]);
-    // a look-ahead transfer into a staging slot may still be in flight; it must have landed before ANY wave writes `ex`
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    if constexpr (ALIASED) {
+        // a look-ahead transfer into the staging slot may still be in flight; it must have landed before ANY wave writes `ex`
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+    }
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
+        const int row = rb * 16 + n;
+        if (row < nrows) {
 #pragma unroll
-        for (int c = 0; c < NOC; ++c) {
+            for (int c = 0; c < NOC; ++c) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) ex.o[wv][rb * 16 + n][out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
-        }
-        if (q == 0) {
-            ex.m[wv][rb * 16 + n] = st.m[rb];
-            ex.l[wv][rb * 16 + n] = st.l[rb];
+                for (int i = 0; i < 4; ++i) ex.o[wv][row][out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
+            }
+            if (q == 0) {
+                ex.m[row][wv] = st.m[rb];
+                ex.l[row][wv] = st.l[rb];
+            }
         }
     }
     __syncthreads();
     HW_MARK(4);
     HW_GLOBAL float* dst = part_o + part * EV;
     constexpr int PASSES = (RB * 16 * EV + NTHREADS * 4 - 1) / (NTHREADS * 4);
+    // every LDS read of every pass is issued before the first value is used: one LDS round trip for the whole combine
+    // (threads beyond the last row read row 0 and store nothing)
+    f32x4 ov[PASSES][NWAVES], mv[PASSES];
 #pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {   // fixed trip count: the LDS reads of all passes can be in flight together
+    for (int ps = 0; ps < PASSES; ++ps) {
         const int idx = tid * 4 + ps * NTHREADS * 4;
-        if (idx >= nrows * EV) break;
-        const int rr = idx / EV, e = idx - rr * EV;
-        float mm = ex.m[0][rr];
+        const int rr = idx < nrows * EV ? idx / EV : 0, e = idx % EV;
+        mv[ps] = *reinterpret_cast<const f32x4*>(&ex.m[rr][0]);
 #pragma unroll
-        for (int w2 = 1; w2 < NWAVES; ++w2) mm = fmaxf(mm, ex.m[w2][rr]);
+        for (int w2 = 0; w2 < NWAVES; ++w2) ov[ps][w2] = *reinterpret_cast<const f32x4*>(&ex.o[w2][rr][e]);
+    }
+    static_assert(NWAVES == 4, "a row's references are read as one float4");
+    const int mrow = tid < nrows ? tid : 0;
+    const f32x4 m4 = *reinterpret_cast<const f32x4*>(&ex.m[mrow][0]), l4 = *reinterpret_cast<const f32x4*>(&ex.l[mrow][0]);
+#pragma unroll
+    for (int ps = 0; ps < PASSES; ++ps) {
+        const int idx = tid * 4 + ps * NTHREADS * 4;
+        const float mm = fmaxf(fmaxf(mv[ps][0], mv[ps][1]), fmaxf(mv[ps][2], mv[ps][3]));
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int w2 = 0; w2 < NWAVES; ++w2) acc += ov[ps][w2] * fast_exp2(mv[ps][w2] - mm);
+        if (idx < nrows * EV) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = acc;
+    }
+    if (tid < nrows) {
+        const float mm = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
         float lsum = 0.f;
 #pragma unroll
-        for (int w2 = 0; w2 < NWAVES; ++w2) {
-            const float wgt = fast_exp2(ex.m[w2][rr] - mm);
-            acc += *reinterpret_cast<const f32x4*>(&ex.o[w2][rr][e]) * wgt;
-            lsum += ex.l[w2][rr] * wgt;
-        }
-        *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = acc;
-        if (e == 0) {
-            HW_GLOBAL float* ml = part_ml + (part + rr) * 2;
-            ml[0] = mm;
-            ml[1] = lsum;
-        }
+        for (int w2 = 0; w2 < NWAVES; ++w2) lsum += l4[w2] * fast_exp2(m4[w2] - mm);
+        *reinterpret_cast<HW_GLOBAL f32x2*>(part_ml + (part + tid) * 2) = f32x2{mm, lsum};
     }
 }
 

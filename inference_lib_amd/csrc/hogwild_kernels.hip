@@ -71,14 +71,19 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
     __shared__ __attribute__((aligned(16))) char q_lds[ROWS * G::QSTR];
     __shared__ int lim_lds[ROWS];
     // One K staging slot per tile in flight, each a separate LDS object so that the wait for a slot's incoming
-    // transfers does not extend to the other slots.  The epilogue exchange reuses the memory of slot 0.
+    // transfers does not extend to the other slots.  Kernels that run one workgroup per CU have LDS to spare and give
+    // the epilogue exchange memory of its own, so that a wave can hand over its accumulators the moment it is done; in
+    // the others the exchange reuses the memory of slot 0.
+    constexpr bool EXSEP = MINW == 1 && sizeof(Ex) + (PF > 1 ? 2 : 1) * SBYTES + ROWS * G::QSTR + 1024 <= 160 * 1024;
     union Slot0 {
         char k[SBYTES];
-        Ex ex;
+        char ex[EXSEP ? 16 : sizeof(Ex)];
     };
     __shared__ __attribute__((aligned(16))) Slot0 slot0;
     __shared__ __attribute__((aligned(16))) char slot1[PF > 1 ? SBYTES : 16];
     __shared__ __attribute__((aligned(16))) char slot2[PF > 2 ? SBYTES : 16];
+    __shared__ __attribute__((aligned(16))) char ex_own[EXSEP ? sizeof(Ex) : 16];
+    Ex& ex = *reinterpret_cast<Ex*>(EXSEP ? ex_own : slot0.ex);
     static_assert(PF <= 3, "three staging slots");
 
     const int tid = threadIdx.x;
@@ -171,7 +176,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
                                       (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
         const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
                                       (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
-        fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW);
+        fv = make_view(kp, vp, hkv, L, __builtin_amdgcn_readlane(my_cap, f), G::KROW, G::VROW, reinterpret_cast<unsigned long long>(a.q));
         lt0 = s0 - fb + wv;     // this wave's first tile of the segment (fragment-local)
         lt1 = s1 - fb;
         if constexpr (DEVLEN) lt1 = min(lt1, (L + TILE - 1) / TILE);   // the fragment may be shorter than planned (or empty)
@@ -253,7 +258,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
 
     HW_MARK(3);
     // ---- merge the four waves of the workgroup and store the partial of this workgroup ----
-    store_partials<DT, EV, RB>(st, slot0.ex, wv, n, q, tid, a.part_o, a.part_ml, (size_t)(hkv * a.wgs_per_head + g) * a.R + r0,
+    store_partials<DT, EV, RB, !EXSEP>(st, ex, wv, n, q, tid, a.part_o, a.part_ml, (size_t)(hkv * a.wgs_per_head + g) * a.R + r0,
                                min(ROWS, a.R - r0));
     HW_MARK(5);
 

@@ -308,7 +308,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
         }
     }
 
-    store_partials<DT, EV, RB>(st, slot0.ex, wv, n, q, tid, ph.part_o, ph.part_ml, (size_t)(hkv * ph.nsplit + split) * ph.R + r0,
+    store_partials<DT, EV, RB, true>(st, slot0.ex, wv, n, q, tid, ph.part_o, ph.part_ml, (size_t)(hkv * ph.nsplit + split) * ph.R + r0,
                                min(ROWS, rend - r0));
 }
 
