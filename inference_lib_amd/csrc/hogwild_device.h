@@ -416,26 +416,37 @@ template <> struct Chunk<F16> {
 };
 
 
-// What each wave of a workgroup hands over at the end (row stride padded so that rows land in different banks).
-// The four waves' references and sums of one row lie next to each other: one 16-byte read fetches all of them.
+// What each wave of a workgroup hands over at the end: its accumulators exactly as the registers hold them (16 bytes
+// per lane and accumulator, lane after lane: no bank conflicts, no register shuffling), and per row the four waves'
+// references and sums next to each other (one 16-byte read fetches all of them).
 template <int ROWS, int EV>
 struct Exchange {
-    float o[NWAVES][ROWS][EV + 4];
+    static constexpr int NSLOT = (ROWS / 16) * (EV / 16);   // accumulators (f32x4 per lane) of one wave
+    f32x4 o[NWAVES][NSLOT][64];
     float m[ROWS][NWAVES];
     float l[ROWS][NWAVES];
 };
 
 // Epilogue shared by the attention kernels: every wave hands over its raw accumulators, running max and sum
-// through LDS (one barrier); then all threads combine them with the weights 2^(m_wave - m_max) and store the
-// workgroup's partial coalesced: `nrows` rows starting at partial row index `part` (EV floats per row in part_o,
-// a (max, sum) pair per row in part_ml).  ALIASED: `ex` shares its memory with a K staging slot, so nobody may
-// write it before every wave is done with its tiles; otherwise each wave hands over as soon as it is done, while
-// the slower waves of the workgroup still compute, and only the combine follows the barrier.  Rows beyond `nrows`
-// (MFMA padding) are neither written nor read.
+// through LDS (one barrier; the exchange is bound by LDS bandwidth: ~40 B/clk for one wave's writes, 128 B/clk for the
+// workgroup's reads); then wave w combines accumulators w*NSLOT/4 ... of all four waves with the weights
+// 2^(m_wave - m_max), still in the accumulator layout (row = lane % 16, so the weights are per-lane scalars), and
+// stores its part of the workgroup's partial: `nrows` rows starting at partial row index `part` (EV floats per row
+// in part_o, a (max, sum) pair per row in part_ml).  A wave's accumulators are consecutive 16-wide chunks of the head
+// dimension whose elements interleave (out_ev), so a lane's values of SPW chunks form runs of SPW consecutive floats.
+// The epilogue runs with one wave per SIMD, i.e. at the issue rate of a single wave: it is written for few
+// instructions, not for few bytes.
+// ALIASED: `ex` shares its memory with a K staging slot, so nobody may write it before every wave is done with its
+// tiles; otherwise each wave hands over as soon as it is done, while the slower waves of the workgroup still compute.
+// Rows beyond `nrows` (MFMA padding) are neither written nor read.
 template <class DT, int EV, int RB, bool ALIASED>
 __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Exchange<RB * 16, EV>& ex, int wv, int n, int q, int tid,
                                                HW_GLOBAL float* part_o, HW_GLOBAL float* part_ml, size_t part, int nrows) {
     constexpr int NOC = EV / 16;
+    constexpr int NSLOT = RB * NOC;
+    constexpr int SPW = NSLOT / NWAVES;       // accumulators each wave combines
+    static_assert(NWAVES == 4 && NSLOT % NWAVES == 0 && NOC % SPW == 0 && SPW <= 4, "a wave's share lies within one row block");
+    const int lane = tid & 63;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) st.l[rb] = quarter_sum(st.l[rb]);
     if constexpr (ALIASED) {
@@ -448,10 +459,7 @@ __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Excha
         const int row = rb * 16 + n;
         if (row < nrows) {
 #pragma unroll
-            for (int c = 0; c < NOC; ++c) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) ex.o[wv][row][out_ev<DT, EV>(c, 4 * q + i)] = st.o[rb][c][i];
-            }
+            for (int c = 0; c < NOC; ++c) ex.o[wv][rb * NOC + c][lane] = st.o[rb][c];
             if (q == 0) {
                 ex.m[row][wv] = st.m[rb];
                 ex.l[row][wv] = st.l[rb];
@@ -460,37 +468,43 @@ __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Excha
     }
     __syncthreads();
     HW_MARK(4);
-    HW_GLOBAL float* dst = part_o + part * EV;
-    constexpr int PASSES = (RB * 16 * EV + NTHREADS * 4 - 1) / (NTHREADS * 4);
-    // every LDS read of every pass is issued before the first value is used: one LDS round trip for the whole combine
-    // (threads beyond the last row read row 0 and store nothing)
-    f32x4 ov[PASSES][NWAVES], mv[PASSES];
+    const int s0 = wv * SPW;                  // first accumulator of this wave's share
+    const int rb = s0 / NOC, c0 = s0 % NOC;
+    const int row = rb * 16 + n;
+    if (row < nrows) {
+        const f32x4 m4 = *reinterpret_cast<const f32x4*>(&ex.m[row][0]);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&ex.l[row][0]);
+        f32x4 ov[SPW][NWAVES];
 #pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-        const int idx = tid * 4 + ps * NTHREADS * 4;
-        const int rr = idx < nrows * EV ? idx / EV : 0, e = idx % EV;
-        mv[ps] = *reinterpret_cast<const f32x4*>(&ex.m[rr][0]);
+        for (int j = 0; j < SPW; ++j)
 #pragma unroll
-        for (int w2 = 0; w2 < NWAVES; ++w2) ov[ps][w2] = *reinterpret_cast<const f32x4*>(&ex.o[w2][rr][e]);
-    }
-    static_assert(NWAVES == 4, "a row's references are read as one float4");
-    const int mrow = tid < nrows ? tid : 0;
-    const f32x4 m4 = *reinterpret_cast<const f32x4*>(&ex.m[mrow][0]), l4 = *reinterpret_cast<const f32x4*>(&ex.l[mrow][0]);
-#pragma unroll
-    for (int ps = 0; ps < PASSES; ++ps) {
-        const int idx = tid * 4 + ps * NTHREADS * 4;
-        const float mm = fmaxf(fmaxf(mv[ps][0], mv[ps][1]), fmaxf(mv[ps][2], mv[ps][3]));
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int w2 = 0; w2 < NWAVES; ++w2) acc += ov[ps][w2] * fast_exp2(mv[ps][w2] - mm);
-        if (idx < nrows * EV) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = acc;
-    }
-    if (tid < nrows) {
+            for (int w2 = 0; w2 < NWAVES; ++w2) ov[j][w2] = ex.o[w2][s0 + j][lane];
         const float mm = fmaxf(fmaxf(m4[0], m4[1]), fmaxf(m4[2], m4[3]));
-        float lsum = 0.f;
+        float wgt[NWAVES];
 #pragma unroll
-        for (int w2 = 0; w2 < NWAVES; ++w2) lsum += l4[w2] * fast_exp2(m4[w2] - mm);
-        *reinterpret_cast<HW_GLOBAL f32x2*>(part_ml + (part + tid) * 2) = f32x2{mm, lsum};
+        for (int w2 = 0; w2 < NWAVES; ++w2) wgt[w2] = fast_exp2(m4[w2] - mm);
+        HW_GLOBAL float* dst = part_o + (part + row) * EV;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float run[SPW];
+#pragma unroll
+            for (int j = 0; j < SPW; ++j) {
+                float acc = ov[j][0][i] * wgt[0];
+#pragma unroll
+                for (int w2 = 1; w2 < NWAVES; ++w2) acc = __builtin_fmaf(ov[j][w2][i], wgt[w2], acc);
+                run[j] = acc;
+            }
+            HW_GLOBAL float* d = dst + out_ev<DT, EV>(c0, 4 * q + i);    // chunks c0 .. c0+SPW-1 are consecutive floats from here
+            if constexpr (SPW == 4) *reinterpret_cast<HW_GLOBAL f32x4*>(d) = f32x4{run[0], run[1], run[2], run[3]};
+            else if constexpr (SPW == 2) *reinterpret_cast<HW_GLOBAL f32x2*>(d) = f32x2{run[0], run[1]};
+            else *d = run[0];
+        }
+        if (q == 0 && c0 == 0) {
+            float lsum = 0.f;
+#pragma unroll
+            for (int w2 = 0; w2 < NWAVES; ++w2) lsum = __builtin_fmaf(l4[w2], wgt[w2], lsum);
+            *reinterpret_cast<HW_GLOBAL f32x2*>(part_ml + (part + row) * 2) = f32x2{mm, lsum};
+        }
     }
 }
 
