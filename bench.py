@@ -8,14 +8,22 @@ on the CPU from a fixed seed and resident in HBM before the timed region starts.
 Cold-cache protocol: the K/V fragments exist in a ring of distinct copies totalling > 640 MB, and
 consecutive steps walk the ring, so neither the L2 nor the 256 MiB Infinity Cache can serve a repeat.
 
-Prints ONE JSON line.  `value` = algorithmic KV bytes per step / measured time per step, where the K
-steps are replayed from one HIP graph (launch overhead of a Python loop would otherwise dominate a
-~10 us step); the eager-loop figure, the hot-cache figure and a plain streaming-read calibration are
-reported under "extra".
+Timing: the K steps (--steps) are captured as one HIP graph (launch overhead of a Python loop would
+otherwise dominate a ~15 us step; the K steps are repeated until the graph holds at least 200) that is
+replayed back to back at least 30 times and at least 2000 steps in total; every replay is bracketed by a
+pair of HIP events on the stream the kernels run on.
+`ms_per_step` is the median over the replays, p10 / p90 are reported next to it, so the figure does not
+depend on --steps.  Before anything is timed the output of the first ring set is checked against the
+CPU reference (the parity gate); the script exits non-zero if it fails.
+
+Prints ONE JSON line.  `value` = algorithmic KV bytes per step / median time per step.  Under "extra":
+the other workload configurations and the paged decode workload measured the same way, the hot-cache
+figure, an eager Python loop, and a plain streaming-read calibration.
 """
 from __future__ import annotations
 
 import argparse
+import ctypes as C
 import json
 import math
 import os
@@ -28,16 +36,9 @@ if ROOT not in sys.path:
 
 PEAK_HBM_GBS = 8000.0   # MI355X published HBM3E bandwidth
 METRIC = "KV-read HBM GB/s (% of peak) + µs/decode step, QwQ-32B shape, 4 workers"
-
-# HBM bytes per launch of the attention kernel measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in
-# separate runs, each scaled by what the same counter reads for the 256 MiB copy kernel this script launches:
-# 0.5 for FETCH_SIZE, 1.0 for WRITE_SIZE): 51.83 MB fetched + 3.03 MB written.  Workloads not measured: None.
-MEASURED_TRAFFIC_BYTES = {"c3_qwq32b_w4": 54_860_000}
-# the same for hw::paged_attention_kernel at the default paged workload (4 x 12528 tokens, blocks of 16): 205.69 MB + 0.67 MB
-MEASURED_PAGED_TRAFFIC_BYTES = {(12528, 16): 206_360_000}
-# packed variable-length workload on the same cache: 383.36 MB fetched (1.87 x the algorithmic bytes: L2 and the Infinity
-# Cache serve most but not all of the 20 row groups' repeats) + 10.92 MB of split-K partials written
-MEASURED_VARLEN_TRAFFIC_BYTES = {(12528, 16): 394_280_000}
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")   # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summaries
+MIN_REPLAYS = 30
+MIN_TOTAL_STEPS = 2000
 
 
 def parse_args():
@@ -47,8 +48,9 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--case", type=int, default=3, help="workload configuration 1..5 (3 = headline)")
     ap.add_argument("--splits", type=int, default=0, help="workgroups per kv head (0 = library default)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (and with it the parity gate)")
     ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only: skip the other configurations under extra")
     ap.add_argument("--ring-mb", type=int, default=640)
     ap.add_argument("--workload", choices=["fragments", "paged", "varlen", "stack"], default="fragments",
                     help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape; "
@@ -61,13 +63,73 @@ def parse_args():
     return ap.parse_args()
 
 
+# ------------------------------------------------------------------------------------------------------------
+# timing
+# ------------------------------------------------------------------------------------------------------------
+def pct(sorted_vals, p):
+    return sorted_vals[min(len(sorted_vals) - 1, max(0, int(round(p * (len(sorted_vals) - 1)))))]
+
+
+MIN_GRAPH_STEPS = 200   # a replay costs a few microseconds of its own: spread over at least this many steps
+
+
+def time_graph(stream, step_fn, K, warmup=20, min_replays=MIN_REPLAYS, min_total=MIN_TOTAL_STEPS):
+    """Capture step_fn(0..K-1) as one HIP graph on `stream` (the K steps repeated until the graph holds at least
+    MIN_GRAPH_STEPS, so that what a replay itself costs does not depend on K), replay it back to back and time every
+    replay with a pair of HIP events recorded on that stream.  Returns microseconds per step: dict(median, p10, p90,
+    replays, graph_steps)."""
+    import torch
+    inner = max(1, math.ceil(MIN_GRAPH_STEPS / K))
+    n = inner * K
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for i in range(n):
+            step_fn(i)
+    replays = max(min_replays, math.ceil(min_total / n))
+    with torch.cuda.stream(stream):
+        for _ in range(max(1, math.ceil(warmup / n))):
+            graph.replay()
+        torch.cuda.synchronize()
+        evs = [torch.cuda.Event(enable_timing=True) for _ in range(replays + 1)]
+        evs[0].record(stream)
+        for r in range(replays):
+            graph.replay()
+            evs[r + 1].record(stream)
+        torch.cuda.synchronize()
+    per = sorted(evs[r].elapsed_time(evs[r + 1]) * 1e3 / n for r in range(replays))
+    del graph
+    return {"median": per[len(per) // 2], "p10": pct(per, 0.10), "p90": pct(per, 0.90), "replays": replays, "graph_steps": n}
+
+
+def load_traffic(key):
+    """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by
+    what the same counter reads for the copy kernel of known size this script launches); None when the workload was
+    not measured.  The numbers live next to the rocprof summaries they come from."""
+    try:
+        with open(TRAFFIC_JSON) as fh:
+            entry = json.load(fh).get(key)
+        return None if entry is None else int(entry["traffic_bytes"])
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+def bench_lib():
+    """The calibration kernels (libhogwild_bench.so, include/hogwild_bench.h); not part of the product library."""
+    path = os.path.join(ROOT, "inference_lib_amd", "libhogwild_bench.so")
+    if not os.path.exists(path):
+        raise SystemExit(f"{path} is missing: build it with `python -m inference_lib_amd.build`")
+    lib = C.CDLL(path)
+    lib.hw_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
+    lib.hw_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    return lib
+
+
 def make_ring(case, dev, ring_mb):
     """Distinct device copies of the KV fragments; q / locations / cos / sin are shared (tiny)."""
     import torch
     kvb = case.kv_bytes()
     n = max(2, math.ceil(ring_mb * 1e6 / kvb))
     ring = []
-    g = torch.Generator().manual_seed(1234)
     for i in range(n):
         if i == 0:
             keys = [k.to(dev) for k in case.keys]
@@ -80,6 +142,132 @@ def make_ring(case, dev, ring_mb):
     return ring
 
 
+class FragmentRun:
+    """One workload configuration set up on the GPU: the ring of KV sets, one prepared hw_problem per set."""
+
+    def __init__(self, case_id, dev, args, with_rq=True):
+        import torch
+        from inference_lib_amd import _lib, cases
+        self.case = case = cases.baseline_case(case_id)
+        self.kv_bytes = case.kv_bytes()
+        self.cd = cd = case.to(dev)
+        self.ring = make_ring(case, dev, args.ring_mb)
+        W, Hq, S, E = cd.q.shape
+        tdt = cd.q.dtype
+        self.out = torch.full((W, Hq, S, E), float("nan"), dtype=tdt, device=dev)
+        self.lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=dev)
+        self.rq = torch.empty((case.F, W, Hq, S, E), dtype=tdt, device=dev) if with_rq else None
+        self.problems = []
+        self.ws = None
+        for keys, vals in self.ring:
+            pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=self.out,
+                              cosines=cd.cos, sines=cd.sin, rq=self.rq, lse=self.lse, splits=args.splits)
+            if self.ws is None:
+                self.ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
+            pr.set_workspace(self.ws)
+            self.problems.append(pr)
+        self.n = len(self.problems)
+        self.plan = _lib.plan(case.lens, W=case.W, S=case.S, Hq=case.Hq, Hkv=case.Hkv, Ev=case.E,
+                              num_cus=_lib.lib.hw_device_cus(), splits=args.splits,
+                              dtype={"f32": _lib.HW_F32, "f16": _lib.HW_F16, "bf16": _lib.HW_BF16}[case.dtype])
+
+    def step(self, i):
+        self.problems[i % self.n].run()
+
+    def kernel(self, i):
+        self.problems[i % self.n].run(stages=1)
+
+    def hot(self, i):
+        self.problems[0].run()
+
+    def name(self):
+        c = self.case
+        return f"W={c.W} S={c.S} Hq={c.Hq} Hkv={c.Hkv} D={c.E} {c.dtype}, fragments={c.lens}"
+
+
+# ------------------------------------------------------------------------------------------------------------
+# parity gate + CPU baseline (the only leg that touches oracle/)
+# ------------------------------------------------------------------------------------------------------------
+def cpu_leg(run, stream):
+    """The reference's eager PyTorch path (python/hogwild/attention.py:38-67 + :84-90) restated in oracle/: first as
+    the checker of the GPU output of ring set 0 (parity gate, exits non-zero on failure), then timed on the host cores
+    of this box as the reported baseline."""
+    import torch
+    from oracle import hogwild_oracle as O
+    case = run.case
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    args = (case.q, case.locations, case.keys, case.values, case.scale, case.cos, case.sin)
+    o_ref, l_ref = O.torch_reference_step(*args)          # fp32 reference on the same (already quantised) inputs
+
+    with torch.cuda.stream(stream):
+        run.out.fill_(float("nan"))
+        run.lse.fill_(float("nan"))
+        run.problems[0].run()
+        torch.cuda.synchronize()
+    got_o, got_l = run.out.float().cpu(), run.lse.cpu()
+    err_o = float((got_o - o_ref).abs().max())
+    err_l = float((got_l - l_ref).abs().max())
+    scale_o = float(o_ref.abs().max())
+    half = case.dtype != "f32"
+    tol_ns = 2e-2 if half else 1e-4                        # the tolerance the task states: max-abs against an fp32 reference
+    tol_o = (2.0 ** -7) * scale_o + 1e-3 if half else 1e-4  # relative to the signal (outputs of a long softmax are small)
+    tol_l = 2e-3 if half else 1e-4
+    ok = bool(torch.isfinite(got_o).all() and torch.isfinite(got_l).all()) and err_o <= min(tol_ns, tol_o) and err_l <= min(tol_ns, tol_l)
+    parity = {"checked": f"out and lse of ring set 0 vs the fp32 CPU reference, {case.dtype}", "max_abs_err_out": err_o,
+              "max_abs_err_lse": err_l, "max_abs_out_ref": scale_o, "tol_out": min(tol_ns, tol_o), "tol_lse": min(tol_ns, tol_l), "ok": ok}
+    if not ok:
+        print(json.dumps({"parity": parity}), file=sys.stderr)
+        print("bench.py: parity gate failed, nothing timed", file=sys.stderr)
+        sys.exit(4)
+
+    for _ in range(2):
+        O.torch_reference_step(*args)
+    ts = []
+    t_all = time.perf_counter()
+    while (len(ts) < 10 or (time.perf_counter() - t_all) < 12.0) and (time.perf_counter() - t_all) < 30.0:   # about 12 s of CPU work
+        t0 = time.perf_counter()
+        O.torch_reference_step(*args)
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    med = ts[len(ts) // 2]
+    baseline = {
+        "value": round(run.kv_bytes / med / 1e9, 3),
+        "unit": "GB/s",
+        "cores": cores,
+        "kind": "port",
+        "us_per_step": round(med * 1e6, 1),
+        "sample": f"{len(ts)} full steps of the same workload (median), torch fp32 eager restatement of the reference path",
+    }
+    return parity, baseline
+
+
+# ------------------------------------------------------------------------------------------------------------
+# workloads
+# ------------------------------------------------------------------------------------------------------------
+def side_config(case_id, dev, args, stream):
+    """Kernel / step time of another workload configuration, measured like the headline (fewer replays)."""
+    import torch
+    run = FragmentRun(case_id, dev, args)
+    K = args.steps
+    kw = dict(warmup=args.warmup, min_replays=10, min_total=1000)
+    with torch.cuda.stream(stream):
+        for i in range(5):
+            run.step(i)
+        torch.cuda.synchronize()
+    step = time_graph(stream, run.step, K, **kw)
+    kern = time_graph(stream, run.kernel, K, **kw)
+    res = {"workload": f"config {case_id} ({run.case.name}): {run.name()}", "kv_bytes_per_step": run.kv_bytes,
+           "workgroups": run.plan.workgroups, "kernel_us": round(kern["median"], 3), "step_us": round(step["median"], 3),
+           "step_us_p10_p90": [round(step["p10"], 3), round(step["p90"], 3)],
+           "kernel_frac_of_peak": round(run.kv_bytes / kern["median"] / 1e3 / PEAK_HBM_GBS, 4),
+           "step_GBps": round(run.kv_bytes / step["median"] / 1e3, 1)}
+    del run
+    torch.cuda.empty_cache()
+    return res
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -88,7 +276,7 @@ def main():
         sys.exit(2)
 
     import torch
-    from inference_lib_amd import _lib, cases
+    from inference_lib_amd import _lib
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -97,182 +285,95 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.workload in ("paged", "varlen"):
-        bench_paged(args, dev)
+        print(json.dumps(bench_paged(args, dev), ensure_ascii=False))
         return
     if args.workload == "stack":
         bench_stack(args, dev)
         return
 
-    case = cases.baseline_case(args.case)
-    kv_bytes = case.kv_bytes()
-    cd = case.to(dev)
-    ring = make_ring(case, dev, args.ring_mb)
+    stream = torch.cuda.Stream()
+    run = FragmentRun(args.case, dev, args, with_rq=not args.no_rq)
+    case, cd, kv_bytes, problems, nring = run.case, run.cd, run.kv_bytes, run.problems, run.n
     W, Hq, S, E = cd.q.shape
     tdt = cd.q.dtype
-
-    out = torch.empty((W, Hq, S, E), dtype=tdt, device=dev)
-    lse = torch.empty((W, Hq, S), dtype=torch.float32, device=dev)
-    rq = None if args.no_rq else torch.empty((case.F, W, Hq, S, E), dtype=tdt, device=dev)
-    problems = []
-    ws = None
-    for keys, vals in ring:
-        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=out,
-                          cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse, splits=args.splits)
-        if ws is None:
-            ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
-        pr.set_workspace(ws)
-        problems.append(pr)
-    nring = len(problems)
-    plan = _lib.plan(case.lens, W=case.W, S=case.S, Hq=case.Hq, Hkv=case.Hkv, Ev=case.E,
-                     num_cus=_lib.lib.hw_device_cus(), splits=args.splits)
-
     K, Wm = args.steps, args.warmup
-    stream = torch.cuda.Stream()
+
+    parity, baseline = (None, None) if args.no_cpu else cpu_leg(run, stream)
+
     with torch.cuda.stream(stream):
         # ---------------- eager loop (launch-bound from Python; reported under extra) ----------------
         for i in range(Wm):
-            problems[i % nring].run()
+            run.step(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(K):
-            problems[i % nring].run()
+            run.step(i)
         torch.cuda.synchronize()
         eager_us = (time.perf_counter() - t0) / K * 1e6
 
-        # ---------------- HIP graph of exactly K steps walking the ring ----------------
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            for i in range(K):
-                problems[i % nring].run()
-        for _ in range(max(1, Wm // max(1, K))):
-            graph.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph.replay()
-        torch.cuda.synchronize()
-        graph_us = (time.perf_counter() - t0) / K * 1e6
+    step = time_graph(stream, run.step, K, warmup=Wm)            # the headline: attention + merge, cold ring
+    kern = time_graph(stream, run.kernel, K, warmup=Wm)          # the attention kernel alone (merge stage off)
+    hot = time_graph(stream, run.hot, K, warmup=Wm, min_replays=10, min_total=1000)
 
-        # ---------------- hot cache: the same KV set every step ----------------
-        graph_hot = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph_hot, stream=stream):
-            for i in range(K):
-                problems[0].run()
-        graph_hot.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph_hot.replay()
-        torch.cuda.synchronize()
-        hot_us = (time.perf_counter() - t0) / K * 1e6
+    # ---------------- the same steps with the fragment lengths read from device memory ----------------
+    len_dev = torch.tensor(case.lens, dtype=torch.int32, device=dev)
+    problems_dl = []
+    for keys, vals in run.ring:
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=run.out,
+                          cosines=cd.cos, sines=cd.sin, rq=run.rq, lse=run.lse, splits=args.splits, len_dev=len_dev)
+        pr.set_workspace(run.ws)
+        problems_dl.append(pr)
+    devlen = time_graph(stream, lambda i: problems_dl[i % nring].run(), K, warmup=Wm, min_replays=10, min_total=1000)
 
-        # ---------------- the same steps with the fragment lengths read from device memory ----------------
-        len_dev = torch.tensor(case.lens, dtype=torch.int32, device=dev)
-        problems_dl = []
-        for keys, vals in ring:
-            pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=out,
-                              cosines=cd.cos, sines=cd.sin, rq=rq, lse=lse, splits=args.splits, len_dev=len_dev)
-            pr.set_workspace(ws)
-            problems_dl.append(pr)
-        graph_dl = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph_dl, stream=stream):
-            for i in range(K):
-                problems_dl[i % nring].run()
-        graph_dl.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        graph_dl.replay()
-        torch.cuda.synchronize()
-        devlen_us = (time.perf_counter() - t0) / K * 1e6
+    # ---------------- the caller-side steps of a decode step at this shape (latency-bound, tiny) ----------------
+    Hkv = cd.keys[0].size(0)
+    seg_k = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
+    seg_v = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
+    k_new = torch.randn((W, S, Hkv, E), device=dev).to(tdt).transpose(1, 2)
+    ck = torch.ones((W, S, E), dtype=tdt, device=dev)
+    inv = torch.ones(E // 2, dtype=torch.float32, device=dev)
+    pos_end = [[1000 + 7 * f + w for w in range(W)] for f in range(case.F)]
+    small = dict(warmup=Wm, min_replays=10, min_total=1000)
+    append = time_graph(stream, lambda i: _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck), K, **small)
+    build = time_graph(stream, lambda i: _lib.build_inputs(pos_end, S, inv, table_dtype=tdt if tdt != torch.float32 else None), K, **small)
 
-        # ---------------- per-launch duration of the attention kernel (HIP events on its stream) ----------------
-        # K launches of the attention kernel alone (merge stage off), replayed as one graph so that the launches
-        # follow each other without host submission gaps, bracketed by two HIP events recorded on this stream.
-        # (An event pair around a single eagerly launched kernel also measures several microseconds of
-        # submission latency; that figure is reported under extra for comparison.)
-        graph_k = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph_k, stream=stream):
-            for i in range(K):
-                problems[i % nring].run(stages=1)
-        graph_k.replay()
-        torch.cuda.synchronize()
-        ea, eb = _lib.Event(), _lib.Event()
-        reps = 3
-        per = []
-        for _ in range(reps):
-            ea.record(stream.cuda_stream)
-            graph_k.replay()
-            eb.record(stream.cuda_stream)
-            torch.cuda.synchronize()
-            per.append(ea.elapsed_ms(eb) * 1e3 / K)
-        kern_us_avg = sum(per) / len(per)
-        kern_us_med = sorted(per)[len(per) // 2]
+    def layer(i):   # what one layer of a decode step launches: key rotation + append, then attention and merge (cold ring)
+        _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck)
+        run.step(i)
+    layer_t = time_graph(stream, layer, K, **small)
 
-        evs2 = [(_lib.Event(), _lib.Event()) for _ in range(K)]
-        for i in range(K):
-            pr = problems[i % nring]
-            pr.set_events(evs2[i][0].handle, evs2[i][1].handle)
-            pr.run()
-            pr.set_events(None, None)
-        torch.cuda.synchronize()
-        d2 = sorted(a.elapsed_ms(b) * 1e3 for a, b in evs2)
-        kern_us_eager_med = d2[len(d2) // 2]
-
-        # ---------------- the caller-side steps of a decode step at this shape (latency-bound, tiny) ----------------
-        Hkv = cd.keys[0].size(0)
-        seg_k = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
-        seg_v = [torch.zeros((Hkv, 256, E), dtype=tdt, device=dev) for _ in range(W)]
-        k_new = torch.randn((W, S, Hkv, E), device=dev).to(tdt).transpose(1, 2)
-        ck = torch.ones((W, S, E), dtype=tdt, device=dev)
-        inv = torch.ones(E // 2, dtype=torch.float32, device=dev)
-        pos_end = [[1000 + 7 * f + w for w in range(W)] for f in range(case.F)]
-        g_a = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g_a, stream=stream):
-            for i in range(K):
-                _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck)
-        g_b = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g_b, stream=stream):
-            for i in range(K):
-                _lib.build_inputs(pos_end, S, inv, table_dtype=tdt if tdt != torch.float32 else None)
-        # what one layer of a decode step launches: key rotation + append, then attention and merge (cold ring)
-        g_c = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g_c, stream=stream):
-            for i in range(K):
-                _lib.rope_append(k_new, k_new, seg_k, seg_v, [i % 200] * W, cosines=ck, sines=ck)
-                problems[i % nring].run()
-        side = []
-        for gr in (g_a, g_b, g_c):
-            gr.replay()
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            gr.replay()
-            torch.cuda.synchronize()
-            side.append((time.perf_counter() - t0) / K * 1e6)
-        append_us, build_us, layer_us = side
-
-        # ---------------- plain streaming read of the whole ring (achievable HBM rate) ----------------
+    # ---------------- plain streaming read of the whole ring (achievable HBM rate) ----------------
+    blib = bench_lib()
+    with torch.cuda.stream(stream):
         big = torch.empty(int(args.ring_mb * 1e6) // 16 * 16, dtype=torch.uint8, device=dev)
         big.random_(0, 255)
         sink = torch.zeros(256, dtype=torch.int32, device=dev)
-        e0, e1 = _lib.Event(), _lib.Event()
-        s_handle = stream.cuda_stream
-        import ctypes as C
+        s_handle = C.c_void_p(stream.cuda_stream)
         for _ in range(2):
-            _lib.check(_lib.lib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), C.c_void_p(s_handle)), "hw_stream_read")
-        e0.record(s_handle)
+            _lib.check(blib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), s_handle), "hw_stream_read")
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
         for _ in range(5):
-            _lib.check(_lib.lib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), C.c_void_p(s_handle)), "hw_stream_read")
-        e1.record(s_handle)
+            _lib.check(blib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), s_handle), "hw_stream_read")
+        e1.record(stream)
         torch.cuda.synchronize()
-        stream_gbs = big.numel() * 5 / (e0.elapsed_ms(e1) * 1e-3) / 1e9
+        stream_gbs = big.numel() * 5 / (e0.elapsed_time(e1) * 1e-3) / 1e9
         # a plain copy of known size (256 MiB read + 256 MiB written): the reference point that scales the
         # FETCH_SIZE / WRITE_SIZE hardware counters when this command runs under rocprofv3 --pmc
         half = 256 * 1024 * 1024
         for _ in range(2):
-            _lib.check(_lib.lib.hw_stream_copy(big.data_ptr() + half, big.data_ptr(), half, C.c_void_p(s_handle)), "hw_stream_copy")
+            _lib.check(blib.hw_stream_copy(big.data_ptr() + half, big.data_ptr(), half, s_handle), "hw_stream_copy")
         torch.cuda.synchronize()
-        del big
+    # launches of the kernel's own byte count walking the same amount of cold memory: what a bare read of these bytes costs
+    kvb16 = kv_bytes // 16 * 16
+    nbare = max(2, big.numel() // kvb16)
+    bare = time_graph(stream, lambda i: _lib.check(blib.hw_stream_read(big.data_ptr() + (i % nbare) * kvb16, kvb16, sink.data_ptr(),
+                                                                       C.c_void_p(stream.cuda_stream)), "hw_stream_read"), K, **small)
+    del big
 
+    graph_us = step["median"]
     value = kv_bytes / (graph_us * 1e-6) / 1e9
-    achieved = kv_bytes / (kern_us_avg * 1e-6) / 1e9
+    achieved = kv_bytes / (kern["median"] * 1e-6) / 1e9
     result = {
         "metric": METRIC,
         "value": round(value, 1),
@@ -287,14 +388,13 @@ def main():
         "dtype": case.dtype,
         "data": "synthetic",
         "config": {
-            "workload": f"config {args.case} ({case.name}): W={case.W} S={case.S} Hq={case.Hq} Hkv={case.Hkv} D={case.E} "
-                        f"{case.dtype}, fragments={case.lens}",
+            "workload": f"config {args.case} ({case.name}): {run.name()}",
             "kv_bytes_per_step": kv_bytes,
             "visible_tokens": case.visible_tokens(),
             "cold_cache_ring_sets": nring,
-            "workgroups": plan.workgroups,
-            "wgs_per_head": plan.wgs_per_head,
-            "writes_rotated_q": rq is not None,
+            "workgroups": run.plan.workgroups,
+            "wgs_per_head": run.plan.wgs_per_head,
+            "writes_rotated_q": run.rq is not None,
         },
         "roofline": {
             "bound": "hbm",
@@ -302,34 +402,59 @@ def main():
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
             "frac": round(achieved / PEAK_HBM_GBS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(case.name),
+            "traffic": load_traffic(f"attention_kernel/{case.name}"),
             "kernel": "hw::attention_kernel",
-            "kernel_us_avg": round(kern_us_avg, 3),
-            "kernel_us_median": round(kern_us_med, 3),
-            "timing": "two HIP events around a graph replay of K attention-kernel launches (merge stage off), divided by K",
+            "kernel_us_avg": round(kern["median"], 3),
+            "kernel_us_p10_p90": [round(kern["p10"], 3), round(kern["p90"], 3)],
+            "timing": f"HIP event pairs around each of {kern['replays']} back-to-back replays of a graph of K attention-kernel launches "
+                      "(merge stage off) on the kernels' stream; median per launch",
         },
         "extra": {
             "us_per_step": round(graph_us, 3),
+            "us_per_step_p10_p90": [round(step["p10"], 3), round(step["p90"], 3)],
+            "graph_replays_timed": step["replays"],
+            "steps_per_graph": step["graph_steps"],
             "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2),
             "eager_loop_us_per_step": round(eager_us, 3),
-            "kernel_us_median_eager_event_pair": round(kern_us_eager_med, 3),
-            "hot_cache_us_per_step": round(hot_us, 3),
-            "device_lengths_us_per_step": round(devlen_us, 3),
-            "hot_cache_GBps": round(kv_bytes / (hot_us * 1e-6) / 1e9, 1),
+            "hot_cache_us_per_step": round(hot["median"], 3),
+            "device_lengths_us_per_step": round(devlen["median"], 3),
+            "hot_cache_GBps": round(kv_bytes / (hot["median"] * 1e-6) / 1e9, 1),
             "stream_read_GBps": round(stream_gbs, 1),
-            "rope_append_us_per_call": round(append_us, 3),
-            "build_inputs_us_per_call": round(build_us, 3),
-            "append_plus_attention_us_per_layer": round(layer_us, 3),
-            "timing": "K steps replayed as one HIP graph, wall clock between device synchronisations",
+            "bare_read_us_per_launch": {"bytes": kvb16, "us": round(bare["median"], 3)},
+            "rope_append_us_per_call": round(append["median"], 3),
+            "build_inputs_us_per_call": round(build["median"], 3),
+            "append_plus_attention_us_per_layer": round(layer_t["median"], 3),
+            "timing": f"K steps captured as one HIP graph, replayed {step['replays']} times back to back, each replay between two HIP "
+                      "events on the kernels' stream; median / p10 / p90 over the replays",
         },
     }
+    if parity is not None:
+        result["extra"]["parity_gate"] = parity
+    else:
+        result["extra"]["parity_gate"] = "skipped (--no-cpu)"
 
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(case, kv_bytes)
+    if not args.no_extra:
+        del run, problems, problems_dl
+        torch.cuda.empty_cache()
+        cfgs = []
+        for cid in (2, 4, 5):
+            if cid != args.case:
+                cfgs.append(side_config(cid, dev, args, stream))
+        pargs = argparse.Namespace(**vars(args))
+        pargs.workload, pargs.no_cpu = "paged", True
+        pg = bench_paged(pargs, dev, quick=True)
+        cfgs.append({"workload": pg["config"]["workload"], "kv_bytes_per_step": pg["config"]["kv_bytes_per_step"],
+                     "workgroups": pg["config"]["workgroups"], "kernel_us": pg["roofline"]["kernel_us_avg"],
+                     "step_us": pg["extra"]["us_per_step"], "step_us_p10_p90": pg["extra"]["us_per_step_p10_p90"],
+                     "kernel_frac_of_peak": pg["roofline"]["frac"], "step_GBps": pg["value"]})
+        result["extra"]["configs"] = cfgs
+
+    if baseline is not None:
+        result["cpu_baseline"] = baseline
     print(json.dumps(result, ensure_ascii=False))
 
 
-def bench_paged(args, dev):
+def bench_paged(args, dev, quick=False):
     """One decode step of hogwild_paged_sdpa: 4 sequences of --seq-len tokens each in a paged bf16 cache (blocks of
     --block-size tokens, shuffled), QwQ-32B head shape, one query token per sequence.  Every sequence has its own KV,
     so a step reads W * seq_len * Hkv * (E + Ev) * 2 bytes.  Cold cache: consecutive steps use block tables that point
@@ -378,6 +503,8 @@ def bench_paged(args, dev):
     plan = _lib.paged_plan(W=W, Hq=Hq, Hkv=Hkv, Ev=D, block_size=bs, max_blocks=nblk, num_cus=_lib.lib.hw_device_cus(), S=S,
                            splits=args.splits, total_q=(q.size(1) if varlen else None))
     K, Wm = args.steps, args.warmup
+    kw = dict(warmup=Wm, min_replays=10, min_total=1000) if quick else dict(warmup=Wm)
+    small = dict(warmup=Wm, min_replays=10, min_total=1000)
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         for i in range(Wm):
@@ -388,46 +515,17 @@ def bench_paged(args, dev):
             problems[i % nring].run()
         torch.cuda.synchronize()
         eager_us = (time.perf_counter() - t0) / K * 1e6
-
-        def graph_of(fn):
-            gr = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(gr, stream=stream):
-                for i in range(K):
-                    fn(i)
-            gr.replay()
-            torch.cuda.synchronize()
-            return gr
-
-        g_step = graph_of(lambda i: problems[i % nring].run())
-        t0 = time.perf_counter()
-        g_step.replay()
-        torch.cuda.synchronize()
-        graph_us = (time.perf_counter() - t0) / K * 1e6
-        g_hot = graph_of(lambda i: problems[0].run())
-        t0 = time.perf_counter()
-        g_hot.replay()
-        torch.cuda.synchronize()
-        hot_us = (time.perf_counter() - t0) / K * 1e6
-        g_k = graph_of(lambda i: problems[i % nring].run(stages=1))
-        ea, eb = _lib.Event(), _lib.Event()
-        per = []
-        for _ in range(3):
-            ea.record(stream.cuda_stream)
-            g_k.replay()
-            eb.record(stream.cuda_stream)
-            torch.cuda.synchronize()
-            per.append(ea.elapsed_ms(eb) * 1e3 / K)
-        kern_us = sum(per) / len(per)
-
+    step = time_graph(stream, lambda i: problems[i % nring].run(), K, **kw)
+    kern = time_graph(stream, lambda i: problems[i % nring].run(stages=1), K, **kw)
+    hot_us = copy_us = None
+    if not quick:
+        hot_us = time_graph(stream, lambda i: problems[0].run(), K, **small)["median"]
         # the append that precedes every decode step: one new token per sequence into the paged cache
         ks = torch.randn((W, 1, Hkv, D), device=dev).to(torch.bfloat16).transpose(1, 2)
         seq = torch.full((W,), L - 1, dtype=torch.int32, device=dev)
-        g_c = graph_of(lambda i: _lib.copy_to_blocks(ks, ks, kc, vc, tables[i % nring], seq))
-        t0 = time.perf_counter()
-        g_c.replay()
-        torch.cuda.synchronize()
-        copy_us = (time.perf_counter() - t0) / K * 1e6
+        copy_us = time_graph(stream, lambda i: _lib.copy_to_blocks(ks, ks, kc, vc, tables[i % nring], seq), K, **small)["median"]
 
+    graph_us, kern_us = step["median"], kern["median"]
     value = kv_bytes / (graph_us * 1e-6) / 1e9
     achieved = kv_bytes / (kern_us * 1e-6) / 1e9
     result = {
@@ -440,13 +538,17 @@ def bench_paged(args, dev):
                                 f"paged decode: W={W} sequences x {L} tokens, S={S}, ") + f"Hq={Hq} Hkv={Hkv} D={D} bf16, block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": (MEASURED_VARLEN_TRAFFIC_BYTES if varlen else MEASURED_PAGED_TRAFFIC_BYTES).get((L, bs)),
+                     "frac": round(achieved / PEAK_HBM_GBS, 4),
+                     "traffic": load_traffic(("paged_attention_kernel/varlen" if varlen else "paged_attention_kernel/decode") + f"_{L}_{bs}"),
                      "kernel": "hw::paged_attention_kernel",
                      "kernel_us_avg": round(kern_us, 3),
-                     "timing": "two HIP events around a graph replay of K attention-kernel launches (merge stage off), divided by K"},
-        "extra": {"us_per_step": round(graph_us, 3), "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2),
-                  "eager_loop_us_per_step": round(eager_us, 3), "hot_cache_us_per_step": round(hot_us, 3),
-                  "copy_to_blocks_us": round(copy_us, 3)},
+                     "kernel_us_p10_p90": [round(kern["p10"], 3), round(kern["p90"], 3)],
+                     "timing": f"HIP event pairs around each of {kern['replays']} back-to-back replays of a graph of K attention-kernel launches "
+                               "(merge stage off); median per launch"},
+        "extra": {"us_per_step": round(graph_us, 3), "us_per_step_p10_p90": [round(step["p10"], 3), round(step["p90"], 3)],
+                  "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2), "eager_loop_us_per_step": round(eager_us, 3),
+                  "hot_cache_us_per_step": None if hot_us is None else round(hot_us, 3),
+                  "copy_to_blocks_us": None if copy_us is None else round(copy_us, 3)},
     }
     if not args.no_cpu:
         from oracle import paged_oracle as po
@@ -467,7 +569,9 @@ def bench_paged(args, dev):
         result["cpu_baseline"] = {"value": round(kv_bytes / med / 1e9, 3), "unit": "GB/s", "cores": cores, "kind": "port",
                                   "us_per_step": round(med * 1e6, 1),
                                   "sample": f"{len(ts)} full steps of the same workload (median), numpy fp32 restatement of the paged kernel"}
-    print(json.dumps(result, ensure_ascii=False))
+    del problems, kc, vc
+    torch.cuda.empty_cache()
+    return result
 
 
 def bench_stack(args, dev):
@@ -560,35 +664,6 @@ def bench_stack(args, dev):
 def np_f32():
     import numpy as np
     return np.float32
-
-
-def cpu_baseline(case, kv_bytes):
-    """The reference's eager PyTorch path (python/hogwild/attention.py:38-67 + :84-90) restated in
-    oracle/, timed on the host cores of this box.  Baseline only."""
-    import torch
-    from oracle import hogwild_oracle as O
-    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
-    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    torch.set_num_threads(cores)
-    args = (case.q, case.locations, case.keys, case.values, case.scale, case.cos, case.sin)
-    for _ in range(2):
-        O.torch_reference_step(*args)
-    ts = []
-    t_all = time.perf_counter()
-    while (len(ts) < 10 or (time.perf_counter() - t_all) < 12.0) and (time.perf_counter() - t_all) < 30.0:   # about 12 s of CPU work
-        t0 = time.perf_counter()
-        O.torch_reference_step(*args)
-        ts.append(time.perf_counter() - t0)
-    ts.sort()
-    med = ts[len(ts) // 2]
-    return {
-        "value": round(kv_bytes / med / 1e9, 3),
-        "unit": "GB/s",
-        "cores": cores,
-        "kind": "port",
-        "us_per_step": round(med * 1e6, 1),
-        "sample": f"{len(ts)} full steps of the same workload (median), torch fp32 eager restatement of the reference path",
-    }
 
 
 if __name__ == "__main__":

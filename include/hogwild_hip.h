@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define HW_ABI_VERSION 3
+#define HW_ABI_VERSION 4
 #define HW_MAX_FRAGMENTS 64
 #define HW_MAX_SPLITS 256      /* workgroups per kv head */
 
@@ -85,8 +85,6 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
  *              spread over more workgroups that read the same KV)
- *   ev_start / ev_stop   optional hipEvent_t recorded on `stream` immediately before / after the attention
- *                        kernel (not the merge kernel); pass NULL outside of profiling
  */
 typedef struct hw_problem {
     int32_t dtype;
@@ -106,8 +104,6 @@ typedef struct hw_problem {
     size_t workspace_bytes;
     int32_t splits;
     int32_t row_blocks;
-    void* ev_start;
-    void* ev_stop;
     const int32_t* cap;
     const int32_t* len_dev;
 } hw_problem;
@@ -332,19 +328,6 @@ int hw_rope_append(const hw_append* a, void* stream);
 
 /* Number of compute units of the current device (0 on failure). */
 int hw_device_cus(void);
-
-/* Small HIP-event helpers so a profiling harness needs no other HIP binding. */
-int hw_event_create(void** ev);
-int hw_event_destroy(void* ev);
-int hw_event_record(void* ev, void* stream);
-int hw_event_synchronize(void* ev);
-int hw_event_elapsed_ms(void* start, void* stop, float* ms);
-
-/* Streaming read of `bytes` bytes (multiple of 16) from `src`, xor-reduced into sink[0..255]: the plain
-   bandwidth calibration the attention kernel is compared with. */
-int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
-/* Plain copy kernel of known size, used to scale FETCH_SIZE / WRITE_SIZE counters. */
-int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -24,8 +24,6 @@ _DTYPE_CODE = {torch.float32: HW_F32, torch.float16: HW_F16, torch.bfloat16: HW_
 EXPORTS = [
     "hw_version", "hw_status_string", "hw_validate", "hw_plan_debug", "hw_workspace_bytes",
     "hw_fused_attention", "hw_fused_attention_stages", "hw_sdpa", "hw_rope", "hw_device_cus",
-    "hw_event_create", "hw_event_destroy", "hw_event_record", "hw_event_synchronize", "hw_event_elapsed_ms",
-    "hw_stream_read", "hw_stream_copy",
     "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
     "hw_paged_sdpa_stages", "hw_copy_to_blocks", "hw_build_inputs", "hw_rope_append",
     "hw_build_inputs_dev", "hw_advance_lengths", "hw_fused_attention_static",
@@ -43,7 +41,6 @@ class HwProblem(C.Structure):
         ("k", C.POINTER(C.c_void_p)), ("v", C.POINTER(C.c_void_p)), ("len", C.POINTER(C.c_int32)),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
         ("splits", C.c_int32), ("row_blocks", C.c_int32),
-        ("ev_start", C.c_void_p), ("ev_stop", C.c_void_p),
         ("cap", C.POINTER(C.c_int32)),
         ("len_dev", C.c_void_p),
     ]
@@ -136,13 +133,6 @@ def _load() -> C.CDLL:
     lib.hw_fused_attention_stages.argtypes = [C.POINTER(HwProblem), C.c_void_p, C.c_int]
     lib.hw_rope.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_int,
                             C.c_int, C.c_int, C.c_int, C.c_void_p]
-    lib.hw_event_create.argtypes = [C.POINTER(C.c_void_p)]
-    lib.hw_event_destroy.argtypes = [C.c_void_p]
-    lib.hw_event_record.argtypes = [C.c_void_p, C.c_void_p]
-    lib.hw_event_synchronize.argtypes = [C.c_void_p]
-    lib.hw_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
-    lib.hw_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
-    lib.hw_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     lib.hw_paged_validate.argtypes = [C.POINTER(HwPagedProblem)]
     lib.hw_paged_plan_debug.argtypes = [C.POINTER(HwPagedProblem), C.c_int, C.POINTER(HwPagedPlan)]
     lib.hw_paged_workspace_bytes.argtypes = [C.POINTER(HwPagedProblem), C.POINTER(C.c_size_t)]
@@ -307,10 +297,6 @@ class Problem:
         self._ws = ws
         self.p.workspace = ws.data_ptr()
         self.p.workspace_bytes = ws.numel() * ws.element_size()
-
-    def set_events(self, start: Optional[int], stop: Optional[int]) -> None:
-        self.p.ev_start = start
-        self.p.ev_stop = stop
 
     def run(self, stages: int = 3) -> None:
         """stages: 1 = attention kernel only (partials stay in the workspace), 2 = merge only, 3 = both."""
@@ -738,29 +724,3 @@ def rope(q: torch.Tensor, cosines: torch.Tensor, sines: torch.Tensor, out: torch
         check(lib.hw_rope(out.data_ptr(), q.data_ptr(), cosines.data_ptr(), sines.data_ptr(), _DTYPE_CODE[out.dtype],
                           F, W, Hq, S, E, rot, C.c_void_p(stream)), "hw_rope")
     return out
-
-
-class Event:
-    """A HIP event created through the library (for per-kernel timing on the op's own stream)."""
-
-    def __init__(self):
-        h = C.c_void_p()
-        check(lib.hw_event_create(C.byref(h)), "hw_event_create")
-        self.handle = h.value
-
-    def record(self, stream: int) -> None:
-        check(lib.hw_event_record(self.handle, C.c_void_p(stream)), "hw_event_record")
-
-    def synchronize(self) -> None:
-        check(lib.hw_event_synchronize(self.handle), "hw_event_synchronize")
-
-    def elapsed_ms(self, stop: "Event") -> float:
-        ms = C.c_float()
-        check(lib.hw_event_elapsed_ms(self.handle, stop.handle, C.byref(ms)), "hw_event_elapsed_ms")
-        return ms.value
-
-    def __del__(self):
-        try:
-            lib.hw_event_destroy(self.handle)
-        except Exception:
-            pass

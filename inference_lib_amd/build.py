@@ -2,6 +2,7 @@
 
   libhogwild_hip.so ... HIP kernels + the C ABI declared in include/hogwild_hip.h
   hogatt.abi3.so ...... torch operator binding (namespace libhogatt) on top of the C ABI
+  libhogwild_bench.so . calibration kernels of the measurement harness (include/hogwild_bench.h), not part of the product
 
 Run as `python -m inference_lib_amd.build`.  hipcc cross-compiles for gfx950 without a GPU present.
 """
@@ -17,6 +18,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhogwild_hip.so")
 TORCH_EXT = os.path.join(HERE, "hogatt.abi3.so")
+BENCH_LIB = os.path.join(HERE, "libhogwild_bench.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -37,6 +39,13 @@ def build_library() -> str:
            "-munsafe-fp-atomics", *DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *srcs]
     _run(cmd)
     return LIB
+
+
+def build_bench_library() -> str:
+    cmd = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc", *DEVICE_FLAGS,
+           "-I", os.path.join(ROOT, "include"), "-o", BENCH_LIB, os.path.join(CSRC, "hogwild_bench.hip")]
+    _run(cmd)
+    return BENCH_LIB
 
 
 def build_torch_binding() -> str:
@@ -71,6 +80,7 @@ def build_c_example() -> str:
 
 def build_all(with_torch: bool = True) -> None:
     build_library()
+    build_bench_library()
     build_c_example()
     if with_torch:
         build_torch_binding()

@@ -241,16 +241,8 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
 
     hipError_t e = hipSuccess;
     if (stages & HW_STAGE_ATTENTION) {
-    if (p->ev_start != nullptr) {
-        e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_start), stream);
+        e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, stream);
         if (e != hipSuccess) return (int)e;
-    }
-    e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, stream);
-    if (e != hipSuccess) return (int)e;
-    if (p->ev_stop != nullptr) {
-        e = hipEventRecord(reinterpret_cast<hipEvent_t>(p->ev_stop), stream);
-        if (e != hipSuccess) return (int)e;
-    }
     }
     if (!(stages & HW_STAGE_MERGE)) return (int)e;
     hw::MergeArgs ma;
@@ -684,36 +676,6 @@ int hw_rope_append(const hw_append* a, void* stream) { return rope_append_run(a,
 int hw_device_cus(void) {
     int c = 0;
     return device_cus(&c) == HW_OK ? c : 0;
-}
-
-int hw_event_create(void** ev) {
-    if (ev == nullptr) return HW_ERR_NULL;
-    hipEvent_t e;
-    hipError_t r = hipEventCreate(&e);
-    if (r != hipSuccess) return (int)r;
-    *ev = e;
-    return HW_OK;
-}
-int hw_event_destroy(void* ev) { return ev ? (int)hipEventDestroy(reinterpret_cast<hipEvent_t>(ev)) : HW_ERR_NULL; }
-int hw_event_record(void* ev, void* stream) {
-    return ev ? (int)hipEventRecord(reinterpret_cast<hipEvent_t>(ev), reinterpret_cast<hipStream_t>(stream)) : HW_ERR_NULL;
-}
-int hw_event_synchronize(void* ev) { return ev ? (int)hipEventSynchronize(reinterpret_cast<hipEvent_t>(ev)) : HW_ERR_NULL; }
-int hw_event_elapsed_ms(void* start, void* stop, float* ms) {
-    if (!start || !stop || !ms) return HW_ERR_NULL;
-    return (int)hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(stop));
-}
-
-int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream) {
-    if (src == nullptr || sink == nullptr) return HW_ERR_NULL;
-    if (bytes % 16 != 0 || !aligned16(src)) return HW_ERR_ALIGN;
-    return (int)hw::launch_stream_read(src, bytes, sink, reinterpret_cast<hipStream_t>(stream));
-}
-
-int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream) {
-    if (src == nullptr || dst == nullptr) return HW_ERR_NULL;
-    if (bytes % 16 != 0 || !aligned16(src) || !aligned16(dst)) return HW_ERR_ALIGN;
-    return (int)hw::launch_stream_copy(dst, src, bytes, reinterpret_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

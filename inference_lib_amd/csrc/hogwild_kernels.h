@@ -65,8 +65,6 @@ hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipS
 hipError_t launch_merge(const MergeArgs& ma, int dtype, int EV, hipStream_t stream);
 hipError_t launch_rope(void* out, const void* q, const float* cosv, const float* sinv, int dtype, int F, int W, int Hq, int S,
                        int E, int RotE, hipStream_t stream);
-hipError_t launch_stream_read(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream);
-hipError_t launch_stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream);
 
 // ---- paged variants: KV of worker w lives in blocks of a shared cache, found through a block table ----
 

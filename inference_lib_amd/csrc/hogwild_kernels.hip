@@ -397,20 +397,6 @@ __global__ __launch_bounds__(256) void rope_kernel(void* out_, const void* q_, c
     }
 }
 
-__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, size_t n16, u32* sink) {
-    u32x4 acc = {0, 0, 0, 0};
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) {
-        u32x4 x = __builtin_nontemporal_load(src + i);
-        acc ^= x;
-    }
-    u32 r = acc.x ^ acc.y ^ acc.z ^ acc.w;
-    if (r == 0x9e3779b9u) sink[threadIdx.x] = r;   // practically never: keeps the loads alive without a store stream
-}
-
-__global__ __launch_bounds__(256) void stream_copy_kernel(u32x4* dst, const u32x4* src, size_t n16) {
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) dst[i] = src[i];
-}
-
 // ------------------------------------------------------------------------------------------------
 // launchers
 // ------------------------------------------------------------------------------------------------
@@ -478,17 +464,6 @@ hipError_t launch_rope(void* out, const void* q, const float* cosv, const float*
         case 1: hipLaunchKernelGGL((rope_kernel<F16>), dim3(blocks), dim3(256), 0, stream, out, q, cosv, sinv, F, W, Hq, S, E, RotE); break;
         default: hipLaunchKernelGGL((rope_kernel<BF16>), dim3(blocks), dim3(256), 0, stream, out, q, cosv, sinv, F, W, Hq, S, E, RotE); break;
     }
-    return hipGetLastError();
-}
-
-hipError_t launch_stream_read(const void* src, size_t bytes, uint32_t* sink, hipStream_t stream) {
-    hipLaunchKernelGGL(stream_read_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<const u32x4*>(src), bytes / 16, sink);
-    return hipGetLastError();
-}
-
-hipError_t launch_stream_copy(void* dst, const void* src, size_t bytes, hipStream_t stream) {
-    hipLaunchKernelGGL(stream_copy_kernel, dim3(2048), dim3(256), 0, stream, reinterpret_cast<u32x4*>(dst),
-                       reinterpret_cast<const u32x4*>(src), bytes / 16);
     return hipGetLastError();
 }
 

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
     for name in declared:
         assert hasattr(L.lib, name), name
-    assert L.lib.hw_version() == 3
+    assert L.lib.hw_version() == 4
 
 
 def test_struct_layout_matches_header():
@@ -36,7 +36,7 @@ def test_struct_layout_matches_header():
     with tempfile.TemporaryDirectory() as d:
         src = os.path.join(d, "s.c")
         open(src, "w").write('#include <stdio.h>\n#include <stddef.h>\n#include "hogwild_hip.h"\nint main(){printf("%zu %zu %zu %zu %zu\\n",'
-                             'sizeof(hw_problem),sizeof(hw_plan),offsetof(hw_problem,workspace),offsetof(hw_problem,ev_start),'
+                             'sizeof(hw_problem),sizeof(hw_plan),offsetof(hw_problem,workspace),offsetof(hw_problem,len_dev),'
                              'offsetof(hw_plan,workspace_bytes));return 0;}\n')
         exe = os.path.join(d, "s")
         subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), src, "-o", exe], check=True)
@@ -44,7 +44,7 @@ def test_struct_layout_matches_header():
     assert int(out[0]) == C.sizeof(L.HwProblem)
     assert int(out[1]) == C.sizeof(L.HwPlan)
     assert int(out[2]) == L.HwProblem.workspace.offset
-    assert int(out[3]) == L.HwProblem.ev_start.offset
+    assert int(out[3]) == L.HwProblem.len_dev.offset
     assert int(out[4]) == L.HwPlan.workspace_bytes.offset
 
 
