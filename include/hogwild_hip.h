@@ -11,7 +11,7 @@
  *   hw_sdpa ................ hogwild_attention        src/binding.cu:255-267, :39-108 (schema :363-364)
  *                            + launcher v21::hogwild_attention_gpu, src/kernels/kernel_v21.cuh:951-996
  *   hw_rope ................ hogwild_rope             src/binding.cu:298-308, :217-253; src/rope.cuh:54-62
- *   hw_workspace_bytes ..... the launcher's private workspace sizing, src/kernels/kernel_v21.cuh:969-980
+ *   hw_workspace_bytes, hw_sdpa_workspace_bytes ... the launcher's private workspace sizing, src/kernels/kernel_v21.cuh:969-980
  *   hw_problem ............. struct Shape + the launcher argument list, src/common.h:5-20,
  *                            src/kernels/kernel_v21.cuh:951-957
  *   hw_status / hw_status_string ... cudaError_t + CUDA_RETURN_ON_ERROR, src/cuda_check.cuh:6-29
@@ -132,8 +132,11 @@ int hw_validate(const hw_problem* p, int fused);
 /* Host-only: the split plan for a device with `num_cus` compute units. */
 int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan);
 
-/* Workspace size for the current device. */
+/* Workspace size for the current device: what hw_fused_attention needs for this problem (if the rotary width is not
+   the head dimension and p->rq is NULL, that includes room for the rotated queries); enough for hw_sdpa as well. */
 int hw_workspace_bytes(const hw_problem* p, size_t* bytes);
+/* The same for hw_sdpa alone (pre-rotated queries: RotE, cosines, sines and rq are ignored). */
+int hw_sdpa_workspace_bytes(const hw_problem* p, size_t* bytes);
 
 /* Rotate q per fragment in registers and attend; replaces hogwild_fused. */
 int hw_fused_attention(const hw_problem* p, void* stream);

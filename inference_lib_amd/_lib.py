@@ -26,7 +26,7 @@ EXPORTS = [
     "hw_fused_attention", "hw_fused_attention_stages", "hw_sdpa", "hw_rope", "hw_device_cus",
     "hw_paged_validate", "hw_paged_plan_debug", "hw_paged_workspace_bytes", "hw_paged_sdpa", "hw_varlen_paged_sdpa",
     "hw_paged_sdpa_stages", "hw_copy_to_blocks", "hw_build_inputs", "hw_rope_append",
-    "hw_build_inputs_dev", "hw_advance_lengths", "hw_fused_attention_static",
+    "hw_build_inputs_dev", "hw_advance_lengths", "hw_fused_attention_static", "hw_sdpa_workspace_bytes",
 ]
 
 
@@ -127,6 +127,7 @@ def _load() -> C.CDLL:
     lib.hw_validate.argtypes = [C.POINTER(HwProblem), C.c_int]
     lib.hw_plan_debug.argtypes = [C.POINTER(HwProblem), C.c_int, C.POINTER(HwPlan)]
     lib.hw_workspace_bytes.argtypes = [C.POINTER(HwProblem), C.POINTER(C.c_size_t)]
+    lib.hw_sdpa_workspace_bytes.argtypes = [C.POINTER(HwProblem), C.POINTER(C.c_size_t)]
     lib.hw_fused_attention.argtypes = [C.POINTER(HwProblem), C.c_void_p]
     lib.hw_sdpa.argtypes = [C.POINTER(HwProblem), C.c_void_p]
     lib.hw_fused_attention_static.argtypes = [C.POINTER(HwProblem), C.c_void_p]
@@ -288,7 +289,8 @@ class Problem:
     def workspace_bytes(self) -> int:
         n = C.c_size_t(0)
         with torch.cuda.device(self.device):
-            check(lib.hw_workspace_bytes(C.byref(self.p), C.byref(n)), "hw_workspace_bytes")
+            fn = lib.hw_sdpa_workspace_bytes if self.prerotated else lib.hw_workspace_bytes
+            check(fn(C.byref(self.p), C.byref(n)), fn.__name__)
         return n.value
 
     def set_workspace(self, ws: Optional[torch.Tensor] = None) -> None:

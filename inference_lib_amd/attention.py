@@ -57,14 +57,28 @@ def hogwild_fused(queries: torch.Tensor, locations: torch.Tensor, keys: List[tor
     return out
 
 
+def _in_place_or_contiguous(keys: List[torch.Tensor], values: List[torch.Tensor]):
+    ks, vs = [], []
+    for k, v in zip(keys, values):
+        k3, v3 = (k[0] if k.dim() == 4 else k), (v[0] if v.dim() == 4 else v)
+        if k3.dim() == 3 and v3.dim() == 3 and _lib.fragment_capacity(k3, v3) is not None:
+            ks.append(k)
+            vs.append(v)
+        else:
+            ks.append(k.contiguous())
+            vs.append(v.contiguous())
+    return ks, vs
+
+
 def hogwild_sdpa(queries: torch.Tensor, locations: torch.Tensor, keys: List[torch.Tensor], values: List[torch.Tensor],
                  scale: float, fragment_lengths=None, out=None, lse: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention with already-rotated queries [F,W,Hq,S,E] (python/hogwild/attention.py:26-35)."""
     if out is None:
         out = torch.empty((queries.size(1), queries.size(2), queries.size(3), values[0].size(-1)), dtype=queries.dtype,
                           device=queries.device)
-    keys = [k.contiguous() for k in keys]
-    values = [v.contiguous() for v in values]
+    # the reference wrapper makes every fragment contiguous (:32-33); a segment that grows in place inside a larger
+    # allocation (rows contiguous, kv heads a whole number of rows apart) is read where it is instead of being copied
+    keys, values = _in_place_or_contiguous(keys, values)
     if HAVE_TORCH_OPS:
         if fragment_lengths is None:
             fragment_lengths = torch.tensor([k.size(-2) for k in keys], dtype=torch.int32, device=queries.device)

@@ -135,6 +135,9 @@ class HogwildCache:
                 raise ValueError("all layers of a segment must hold the same number of tokens (call between decode steps)")
         if len({id(seg) for seg in self.write_to}) != len(self.write_to):
             raise ValueError("with device-resident lengths every worker needs a segment of its own to write to")
+        if any(seg is not order[-1] for seg, order in zip(self.write_to, self.cache_structure)):
+            # position ids are formed from the last segment of a worker's order (attention.py:238-246) in both modes
+            raise ValueError("with device-resident lengths every worker must write to the last segment of its order")
         n_new = [int(new_tokens)] * len(self.write_to) if n_new is None else [int(x) for x in n_new]
         if len(n_new) != len(self.write_to) or any(x < 0 or x > int(new_tokens) for x in n_new):
             raise ValueError("n_new: one number per worker, between 0 and new_tokens")
@@ -180,9 +183,21 @@ class HogwildCache:
         return min(((b - n) // a for n, b, a in zip(lens, self._dev["bound"], self._dev["add"]) if a > 0), default=0)
 
     def use_host_lengths(self) -> None:
-        """Leave the device-resident-lengths mode (after reading the lengths back)."""
-        self.sync_lengths()
+        """Leave the device-resident-lengths mode (after reading the lengths back).  The mode is left even if the read-back
+        finds an overrun: the host lengths are then clamped to the planned bounds (what was attended to) and the error is
+        raised afterwards."""
+        d = self._dev
+        if d is None:
+            return
         self._dev = None
+        lens = d["len_dev"].tolist()
+        for seg, n, b in zip(d["segments"], lens, d["bound"]):
+            seg.lengths = [int(min(n, b))] * len(seg.lengths)
+        over = [f for f, (n, b) in enumerate(zip(lens, d["bound"])) if n > b]
+        if over:
+            raise RuntimeError(f"segments {over} grew beyond the lengths the steps were planned for ({lens} vs {d['bound']}): "
+                               "the captured step was replayed more often than headroom // new_tokens; the tokens beyond the "
+                               "bounds were dropped")
 
     def _update_dev(self, key_states, value_states, cos, sin, layer_idx, mode) -> CacheStructure:
         d = self._dev
@@ -325,6 +340,7 @@ def merge_caches(target: SegmentCache, source: SegmentCache, model=None, *, inv_
     sin = sin.reshape(1, 1, -1).to(tdt)
     for layer in range(len(target.k)):
         m = source.lengths[layer]
+        target.reserve(layer, m)          # grow like every other append (the reference's merge goes through target.update)
         _lib.rope_append(source.k[layer][:, :m, :].unsqueeze(0), source.v[layer][:, :m, :].unsqueeze(0), [target.k[layer]], [target.v[layer]],
                          [target.lengths[layer]], cosines=cos, sines=sin, mode=mode)
         target.lengths[layer] += m

@@ -152,7 +152,10 @@ void unpack_common(Unpacked& u, at::Tensor& out, double scale, const at::Tensor&
 void run(Unpacked& u, const at::Tensor& out, bool fused) {
     c10::hip::HIPGuardMasqueradingAsCUDA guard(out.device());   // ROCm tensors report the device type "cuda"
     size_t bytes = 0;
-    check_status(hw_workspace_bytes(&u.p, &bytes), "hw_workspace_bytes");
+    if (fused)
+        check_status(hw_workspace_bytes(&u.p, &bytes), "hw_workspace_bytes");
+    else
+        check_status(hw_sdpa_workspace_bytes(&u.p, &bytes), "hw_sdpa_workspace_bytes");
     u.workspace = at::empty({(int64_t)bytes}, out.options().dtype(at::kByte));
     u.p.workspace = u.workspace.data_ptr();
     u.p.workspace_bytes = bytes;

@@ -10,8 +10,11 @@
 
 #include "../../include/hogwild_hip.h"
 #include "hogwild_kernels.h"
+#include "hogwild_plan.h"
 
 namespace {
+
+using namespace hw::host;
 
 constexpr int kMaxDevices = 64;
 std::atomic<int> g_cus[kMaxDevices];   // 0 = not queried yet
@@ -54,132 +57,6 @@ int static_scratch(void** ptr) {
     return HW_OK;
 }
 
-bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-size_t elem_size(int dtype) { return dtype == HW_F32 ? 4 : 2; }
-
-int validate(const hw_problem* p, int fused) {
-    if (p == nullptr) return HW_ERR_NULL;
-    if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
-    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
-    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
-    if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
-    if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return HW_ERR_SHAPE;   // the row max is taken before scaling
-    if (fused) {
-        if (p->RotE < 0 || p->RotE > p->E || (p->RotE & 1)) return HW_ERR_SHAPE;
-    }
-    if (p->out == nullptr || p->q == nullptr || p->locations == nullptr) return HW_ERR_NULL;
-    if (p->k == nullptr || p->v == nullptr || p->len == nullptr) return HW_ERR_NULL;
-    if (fused && p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
-    if (p->len_dev != nullptr && (!fused || p->RotE != p->E)) return HW_ERR_UNSUPPORTED;   // fused entry, full rotary width only
-    long long rows = (long long)p->W * p->S * (p->Hq / p->Hkv);
-    if (rows >= (1 << 20) || p->S >= (1 << 12) || p->Hq / p->Hkv >= (1 << 12)) return HW_ERR_SHAPE;
-    if ((long long)p->Hkv * ((rows + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
-    for (int f = 0; f < p->F; ++f) {
-        if (p->len[f] < 0) return HW_ERR_SHAPE;
-        if (p->cap != nullptr && p->cap[f] < p->len[f]) return HW_ERR_SHAPE;
-        if (p->len[f] > 0 && (p->k[f] == nullptr || p->v[f] == nullptr)) return HW_ERR_NULL;
-        if (!aligned16(p->k[f]) || !aligned16(p->v[f])) return HW_ERR_ALIGN;
-        // one kv head of a fragment is addressed through a 32-bit buffer offset
-        if ((long long)p->len[f] * (p->E > p->Ev ? p->E : p->Ev) * (long long)elem_size(p->dtype) >= 0x7fff0000ll) return HW_ERR_SHAPE;
-    }
-    if (!aligned16(p->out) || !aligned16(p->q)) return HW_ERR_ALIGN;
-    if (fused && (!aligned16(p->cosines) || !aligned16(p->sines) || !aligned16(p->rq))) return HW_ERR_ALIGN;
-    // kernels are instantiated for these head dims (never a silent no-op as in kernel_v21.cuh:992-995)
-    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
-    return HW_OK;
-}
-
-int make_plan(const hw_problem* p, int num_cus, hw_plan* plan) {
-    if (plan == nullptr) return HW_ERR_NULL;
-    if (num_cus < 1) return HW_ERR_SHAPE;
-    std::memset(plan, 0, sizeof(*plan));
-    const int rows = p->W * p->S * (p->Hq / p->Hkv);
-    plan->rows = rows;
-    plan->row_blocks = rows <= 16 ? 1 : 2;
-    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
-    const int rows_per_wg = 16 * plan->row_blocks;
-    plan->row_groups = (rows + rows_per_wg - 1) / rows_per_wg;
-    plan->tile_tokens = hw::TILE;
-    long long tiles = 0;
-    for (int f = 0; f < p->F; ++f) {
-        plan->tile_begin[f] = (int)tiles;
-        tiles += (p->len[f] + hw::TILE - 1) / hw::TILE;
-        if (tiles > (1ll << 30)) return HW_ERR_SHAPE;
-    }
-    for (int f = p->F; f <= HW_MAX_FRAGMENTS; ++f) plan->tile_begin[f] = (int)tiles;
-    plan->tiles_per_head = (int)tiles;
-
-    // Split-K policy: fill every CU with its resident workgroups once, but at least one tile per wave
-    // in every workgroup, and never more workgroups than tiles.
-    int wgs = p->splits;
-    if (wgs <= 0) {
-        // the two-row-block and fp32 kernels are built for one wave per SIMD (one workgroup per CU)
-        const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32) ? 2 : 1;
-        const int target = per_cu * num_cus;
-        wgs = target / (p->Hkv * plan->row_groups);
-        const int by_work = (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
-        if (wgs > by_work) wgs = by_work;
-    }
-    if (wgs > (int)tiles) wgs = (int)tiles;
-    if (wgs > hw::MAX_SPLITS) wgs = hw::MAX_SPLITS;
-    if (wgs < 1) wgs = 1;
-
-    // Workgroup boundaries.  Opening a fragment costs a workgroup a fixed prologue (query rotation, a
-    // barrier, a pipeline refill) worth about kOpenCost tiles, so boundaries balance tiles + openings
-    // rather than tiles alone: a run of tiny fragments is spread over several workgroups instead of
-    // serialising their prologues in one straggler.
-    {
-        const double kOpenCost = 6.0;
-        int nfrag_left = 0;
-        for (int f = 0; f < p->F; ++f) nfrag_left += p->len[f] > 0 ? 1 : 0;
-        long long tiles_left = tiles;
-        int wg = 0;
-        double used = 0.0;
-        plan->wg_tile_begin[0] = 0;
-        for (int f = 0; f < p->F; ++f) {
-            const int ft = (p->len[f] + hw::TILE - 1) / hw::TILE;
-            if (ft == 0) continue;
-            int t = 0;
-            while (t < ft) {
-                const int wgs_left = wgs - wg;   // including the current one
-                // fair share of what remains, counting one opening per remaining fragment and workgroup
-                const double remaining = (double)tiles_left + kOpenCost * (nfrag_left + wgs_left - 1) + used;
-                const double target = remaining / wgs_left;
-                const double room = target - used - kOpenCost;
-                if (room < 1.0 && used > 0.0 && wgs_left > 1) {   // not worth opening this fragment here
-                    plan->wg_tile_begin[++wg] = plan->tile_begin[f] + t;
-                    used = 0.0;
-                    continue;
-                }
-                int take = (int)(room + 0.5);
-                if (take < 1) take = 1;
-                if (take > ft - t || wgs_left == 1) take = ft - t;
-                used += kOpenCost + take;
-                t += take;
-                tiles_left -= take;
-                if (t < ft) {   // the fragment continues in the next workgroup
-                    plan->wg_tile_begin[++wg] = plan->tile_begin[f] + t;
-                    used = 0.0;
-                }
-            }
-            --nfrag_left;
-        }
-        wgs = tiles > 0 ? wg + 1 : 1;
-        for (int i = wgs; i <= HW_MAX_SPLITS; ++i) plan->wg_tile_begin[i] = (int)tiles;
-    }
-    plan->wgs_per_head = wgs;
-    plan->workgroups = wgs * p->Hkv * plan->row_groups;
-    const size_t parts = (size_t)p->Hkv * wgs;
-    plan->workspace_bytes = parts * rows * ((size_t)p->Ev + 2) * sizeof(float);
-    plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
-    // the attention kernel rotates in its prologue only over the full head dimension; any other rotary width
-    // goes through the standalone rotation first, into the caller's rq buffer or, without one, into the workspace
-    if (p->RotE != p->E && p->RotE >= 0)
-        plan->workspace_bytes += ((size_t)p->F * p->W * p->Hq * p->S * p->E * elem_size(p->dtype) + 255) & ~(size_t)255;
-    return HW_OK;
-}
-
 int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATTENTION | HW_STAGE_MERGE) {
     int st = validate(p, fused);
     if (st != HW_OK) return st;
@@ -187,7 +64,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     st = device_cus(&cus);
     if (st != HW_OK) return st;
     hw_plan plan;
-    st = make_plan(p, cus, &plan);
+    st = make_plan(p, cus, &plan, fused);
     if (st != HW_OK) return st;
     if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
 
@@ -233,7 +110,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
     ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
     // multipliers for the in-kernel divisions (exact for numerators < 2^20 and divisors < 2^12, both validated)
-    auto magic = [](int d) { return (unsigned)(((1ull << 32) + (unsigned long long)d - 1) / (unsigned long long)d); };
+    auto magic = [](int d) { return magic_of(d); };
     ka.h.magic_gq = magic(p->Hq / p->Hkv);
     ka.h.magic_s = magic(p->S);
     ka.h.magic_nrg = magic(plan.row_groups);
@@ -260,80 +137,6 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
 // ---------------------------------------------------------------------------------------------------------
 // paged variants
 // ---------------------------------------------------------------------------------------------------------
-int paged_validate(const hw_paged_problem* p) {
-    if (p == nullptr) return HW_ERR_NULL;
-    if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
-    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
-    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
-    if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
-    if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return HW_ERR_SHAPE;
-    const bool varlen = p->cu_seqlens_q != nullptr;
-    if (varlen ? p->total_q < 0 : (p->S < 1 || p->S >= (1 << 12))) return HW_ERR_SHAPE;
-    if (p->block_size < 1 || p->block_size >= (1 << 12) || p->max_blocks < 1 || p->num_blocks < 1) return HW_ERR_SHAPE;
-    if ((long long)p->block_size * p->max_blocks > (1ll << 20)) return HW_ERR_SHAPE;
-    if ((long long)p->num_blocks * p->Hkv * p->block_size >= (1ll << 31)) return HW_ERR_SHAPE;
-    const long long tokens = varlen ? p->total_q : (long long)p->W * p->S;
-    const int gq = p->Hq / p->Hkv;
-    if (gq >= (1 << 12) || tokens * gq >= (1 << 20) || p->W >= (1 << 20)) return HW_ERR_SHAPE;
-    if (p->out == nullptr || p->q == nullptr || p->locations == nullptr || p->fragment_lengths == nullptr) {
-        if (tokens > 0) return HW_ERR_NULL;
-    }
-    if (p->key_cache == nullptr || p->value_cache == nullptr || p->block_table == nullptr) return HW_ERR_NULL;
-    if (!aligned16(p->out) || !aligned16(p->q) || !aligned16(p->key_cache) || !aligned16(p->value_cache)) return HW_ERR_ALIGN;
-    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
-    return HW_OK;
-}
-
-int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
-    if (plan == nullptr) return HW_ERR_NULL;
-    if (num_cus < 1) return HW_ERR_SHAPE;
-    std::memset(plan, 0, sizeof(*plan));
-    const bool varlen = p->cu_seqlens_q != nullptr;
-    const int gq = p->Hq / p->Hkv;
-    const long long tokens = varlen ? p->total_q : (long long)p->W * p->S;
-    plan->rows = (int)(tokens * gq);
-    // rows of one worker share its KV: one 16-row block is enough for plain decoding, two when a worker brings
-    // more rows (several query tokens, wide GQA groups)
-    const long long rows_per_worker = varlen ? (tokens * gq + p->W - 1) / p->W : (long long)p->S * gq;
-    plan->row_blocks = rows_per_worker <= 16 ? 1 : 2;
-    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
-    if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
-    const int rpw = 16 * plan->row_blocks;
-    long long items;
-    if (varlen) items = p->W + tokens * gq / rpw;          // sum_w ceil(rows_w / rpw) <= W + rows / rpw
-    else items = (long long)p->W * (((long long)p->S * gq + rpw - 1) / rpw);
-    if (items < 1) items = 1;
-    plan->row_groups = (int)items;
-    int splits = p->splits;
-    if (splits <= 0) {
-        // The paged kernels run one workgroup per CU.  Few (kv head, row group) pairs: split until every CU has
-        // one workgroup.  More pairs than half the CUs: the chip is oversubscribed anyway, and about three
-        // workgroups per CU even out the tail between sequences of different length (measured best on packed
-        // variable-length queries) -- there a wave keeps at least four tiles.
-        const long long pairs = (long long)p->Hkv * items;
-        const long long tiles = ((long long)p->block_size * p->max_blocks + hw::TILE - 1) / hw::TILE;
-        long long s, by_work;
-        if (2 * pairs <= num_cus) {
-            s = num_cus / pairs;
-            by_work = (tiles + hw::NWAVES - 1) / hw::NWAVES;
-        } else {
-            s = (3LL * num_cus + pairs - 1) / pairs;
-            by_work = tiles / (4 * hw::NWAVES);
-        }
-        if (s > by_work) s = by_work;
-        splits = (int)s;
-    }
-    if (splits > 64) splits = 64;
-    if (splits < 1) splits = 1;
-    plan->splits = splits;
-    const long long wgs = (long long)p->Hkv * items * splits;
-    if (wgs >= (1 << 20)) return HW_ERR_SHAPE;
-    plan->workgroups = (int)wgs;
-    plan->workspace_bytes = (size_t)p->Hkv * splits * (size_t)(plan->rows > 0 ? plan->rows : 1) * ((size_t)p->Ev + 2) * sizeof(float);
-    plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
-    return HW_OK;
-}
-
 int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     int st = paged_validate(p);
     if (st != HW_OK) return st;
@@ -347,7 +150,7 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     const bool varlen = p->cu_seqlens_q != nullptr;
-    auto magic = [](int d) { return (unsigned)(((1ull << 32) + (unsigned long long)d - 1) / (unsigned long long)d); };
+    auto magic = [](int d) { return magic_of(d); };
 
     hw::PagedHeader ph;
     std::memset(&ph, 0, sizeof(ph));
@@ -569,17 +372,22 @@ int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan) {
     return make_plan(p, num_cus, plan);
 }
 
-int hw_workspace_bytes(const hw_problem* p, size_t* bytes) {
+static int workspace_bytes_for(const hw_problem* p, int fused, size_t* bytes) {
     if (bytes == nullptr) return HW_ERR_NULL;
+    if (p == nullptr || p->len == nullptr) return HW_ERR_NULL;
     int cus = 0;
     int st = device_cus(&cus);
     if (st != HW_OK) return st;
     hw_plan plan;
-    st = hw_plan_debug(p, cus, &plan);
+    st = make_plan(p, cus, &plan, fused);
     if (st != HW_OK) return st;
     *bytes = plan.workspace_bytes;
     return HW_OK;
 }
+
+int hw_workspace_bytes(const hw_problem* p, size_t* bytes) { return workspace_bytes_for(p, 1, bytes); }
+
+int hw_sdpa_workspace_bytes(const hw_problem* p, size_t* bytes) { return workspace_bytes_for(p, 0, bytes); }
 
 int hw_fused_attention(const hw_problem* p, void* stream) { return run(p, stream, 1); }
 

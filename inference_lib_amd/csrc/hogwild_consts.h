@@ -1,0 +1,12 @@
+// Compile-time geometry shared by the host-side planner (plain C++, no HIP) and the kernels.
+#pragma once
+
+namespace hw {
+
+constexpr int MAXF = 64;       // fragments per launch (table travels in the kernel arguments)
+constexpr int TILE = 32;       // tokens per wave step
+constexpr int NWAVES = 4;      // waves per workgroup
+constexpr int NTHREADS = NWAVES * 64;
+constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary table below)
+
+}  // namespace hw

@@ -4,13 +4,9 @@
 #include <stddef.h>
 #include <stdint.h>
 
-namespace hw {
+#include "hogwild_consts.h"
 
-constexpr int MAXF = 64;       // fragments per launch (table travels in the kernel arguments)
-constexpr int TILE = 32;       // tokens per wave step
-constexpr int NWAVES = 4;      // waves per workgroup
-constexpr int NTHREADS = NWAVES * 64;
-constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary table below)
+namespace hw {
 
 // Fragment table passed by value in the kernel arguments: no per-call host-to-device copy of a pointer
 // table (the reference does one, src/binding.cu:84-103).

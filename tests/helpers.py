@@ -2,7 +2,30 @@
 import numpy as np
 import torch
 
-TOL = {"f32": 1e-4, "f16": 2e-2, "bf16": 2e-2}   # max-abs tolerance on out and lse vs the fp32/fp64 oracle
+class Tol(float):
+    """A parity bound.  The float value is the bound the task states (max-abs against the fp32/fp64 oracle: bf16 / fp16
+    2e-2, fp32 1e-4).  For the 16-bit types that alone is weak where outputs are small (a softmax over 12 000 keys of
+    N(0,1) values gives |out| ~ 0.015), so assert_close also applies a bound relative to the signal:
+        out: max|d| <= rel * max|reference| + floor        lse: max|d| <= lse
+    and passes only if both hold."""
+
+    def __new__(cls, stated, rel=None, floor=0.0, lse=None):
+        t = super().__new__(cls, stated)
+        t.rel, t.floor, t.lse = rel, floor, lse
+        return t
+
+    def out_bound(self, want: np.ndarray) -> float:
+        if self.rel is None:
+            return float(self)
+        fin = np.isfinite(want)
+        peak = float(np.abs(want[fin]).max()) if fin.any() else 0.0
+        return min(float(self), self.rel * peak + self.floor)
+
+    def lse_bound(self) -> float:
+        return float(self) if self.lse is None else min(float(self), self.lse)
+
+
+TOL = {"f32": Tol(1e-4), "f16": Tol(2e-2, rel=2.0 ** -7, floor=1e-3, lse=2e-3), "bf16": Tol(2e-2, rel=2.0 ** -7, floor=1e-3, lse=2e-3)}
 
 
 def np64(t: torch.Tensor) -> np.ndarray:
@@ -32,6 +55,9 @@ def run_fused(case_dev, *, splits=0, with_rq=True, with_lse=True):
 
 
 def assert_close(name, got: torch.Tensor, want: np.ndarray, tol: float):
+    """max-abs comparison; a Tol also brings the signal-relative bound (names containing "lse" use its lse bound)."""
+    if isinstance(tol, Tol):
+        tol = tol.lse_bound() if "lse" in name else tol.out_bound(np.asarray(want, dtype=np.float64))
     g = np64(got)
     assert g.shape == want.shape, (name, g.shape, want.shape)
     assert np.isfinite(g[np.isfinite(want)]).all(), f"{name}: non-finite values"

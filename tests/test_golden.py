@@ -79,10 +79,14 @@ def test_gpu_reproduces_summary_of_larger_configs(idx):
     out, lse, _ = run_fused(c.to(torch.device("cuda:0")))
     o = np64(out).reshape(-1)
     tol = TOL[c.dtype]
-    assert np.abs(o[s["sample_index"]] - np.array(s["sample_out"])).max() <= tol
-    assert np.abs(np64(lse).reshape(-1)[:8] - np.array(s["sample_lse"])).max() <= tol
-    assert abs(float(np64(lse).mean()) - s["lse_mean"]) <= tol
-    assert abs(float(np.sqrt((o ** 2).sum())) - s["out_l2"]) <= tol * np.sqrt(o.size)
+    # bounds relative to the recorded values: an output that is all zeros (or off by a few percent) fails every one
+    want = np.array(s["sample_out"])
+    t_out = tol.out_bound(np.array([s["out_abs_max"]]))
+    assert np.abs(o[s["sample_index"]] - want).max() <= t_out
+    assert np.abs(np64(lse).reshape(-1)[:8] - np.array(s["sample_lse"])).max() <= tol.lse_bound()
+    assert abs(float(np64(lse).mean()) - s["lse_mean"]) <= tol.lse_bound()
+    assert abs(float(np.sqrt((o ** 2).sum())) - s["out_l2"]) <= 2.0 ** -7 * s["out_l2"]
+    assert abs(float(np.abs(o).max()) - s["out_abs_max"]) <= t_out
 
 
 # ------------------------------------------------------------------------------------------------ paged / cache fixtures

@@ -276,6 +276,38 @@ def test_merge_caches_rerotates_and_appends(dtype):
             assert np.abs(got_k[:, 77:] - want).max() <= ulp and np.mean(got_k[:, 77:] == want) > 0.99
 
 
+def test_merge_caches_grows_a_target_that_is_too_small():
+    """The source holds more rows than the target has room for: the target moves into larger buffers (as every other
+    append does), keeps its rows, and receives the re-rotated source behind them."""
+    from inference_lib_amd import cache
+    from oracle import cache_oracle as co
+    tdt = torch.bfloat16
+    g = torch.Generator().manual_seed(29)
+    layers, Hkv, D = 2, 2, 128
+    f = inv_freq(D)
+    target = cache.SegmentCache(layers, Hkv, D, 40, dtype=tdt, device=DEV)      # 33 of 40 rows used: room for 7
+    source = cache.SegmentCache(layers, Hkv, D, 64, dtype=tdt, device=DEV)      # 50 rows to merge
+    tk, tv, sk, sv = [], [], [], []
+    for layer in range(layers):
+        for seg, n, ks_, vs_ in ((target, 33, tk, tv), (source, 50, sk, sv)):
+            k = torch.randn((1, Hkv, n, D), generator=g).to(tdt)
+            v = torch.randn((1, Hkv, n, D), generator=g).to(tdt)
+            seg.update(k.to(DEV), v.to(DEV), layer)
+            ks_.append(np64(k[0]))
+            vs_.append(np64(v[0]))
+    assert target.k[0].size(1) == 40
+    cache.merge_caches(target, source, inv_freq=torch.from_numpy(f).to(DEV))
+    torch.cuda.synchronize()
+    assert target.get_seq_length() == 83 and target.k[0].size(1) >= 83 and target.k[1].size(1) >= 83
+    for layer in range(layers):
+        want = co.merge_rerotate(sk[layer], 33, f, storage="bf16", mode="eager")
+        got_k, got_v = np64(target.key_cache[layer][0]), np64(target.value_cache[layer][0])
+        assert got_k.shape[1] == 83
+        assert np.array_equal(got_k[:, :33], tk[layer]) and np.array_equal(got_v[:, :33], tv[layer])
+        assert np.array_equal(got_v[:, 33:], sv[layer])
+        assert np.abs(got_k[:, 33:] - want).max() <= 2.0 ** -6 and np.mean(got_k[:, 33:] == want) > 0.99
+
+
 def test_segment_grows_when_full():
     """A segment that runs out of room moves into buffers of twice the size; contents and later appends are unaffected."""
     from inference_lib_amd.cache import SegmentCache

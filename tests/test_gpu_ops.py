@@ -110,3 +110,43 @@ def test_errors_are_loud():
     with pytest.raises(RuntimeError):
         torch.ops.libhogatt.hogwild_sdpa(out, 0.1, c.locations.long(), torch.zeros((2, 1, 2, 1, 128), dtype=torch.bfloat16, device=dev),
                                          torch.tensor(c.lens, dtype=torch.int32, device=dev), c.keys, c.values)
+
+
+def test_reference_import_path_and_call_sequence(oracle):
+    """An unchanged caller: `from hogwild.attention import hogwild_fused` (python/hogwild/attention.py:12-23) and the call
+    sequence of AttentionModule.forward (:325-336) -- buffers shaped as the cache object shapes them (:206-218), fragments
+    as [1, Hkv, L, D] views of segment caches, the fused operator through its wrapper and through torch.ops.libhogatt
+    directly, then the transpose/reshape of :338-339."""
+    import hogwild.attention as ref_api
+    from hogwild.attention import hogwild_fused, hogwild_rope, hogwild_sdpa
+    from inference_lib_amd import cases
+    assert not hasattr(ref_api, "hogwild_sdpa_pt"), "the pure-torch path is test infrastructure, not part of the package"
+    c = cases.small_case(dtype="bf16", W=3, S=1, Hq=12, Hkv=4, E=128, lens=(257, 40, 64, 9, 3, 1, 2), seed=21, with_cur=True)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    segs = [ref_api.SegmentCache(1, c.Hkv, E, L + 4, dtype=cd.q.dtype, device=_dev()) for L in c.lens]
+    for sg, k, v in zip(segs, cd.keys, cd.values):
+        sg.update(k.unsqueeze(0), v.unsqueeze(0), 0)
+    query_states = cd.q
+    frags = torch.tensor(c.lens, dtype=torch.int32, device=_dev())
+    keys = [sg.key_cache[0] for sg in segs]          # views [1, Hkv, L, D] into the segment buffers
+    values = [sg.value_cache[0] for sg in segs]
+    assert keys[0].dim() == 4 and keys[0].size(0) == 1
+    rq = torch.empty((cd.cos.size(0), W, Hq, S, E), dtype=query_states.dtype, device=_dev())                       # :206-211
+    att_buffer = torch.empty((rq.size(1), rq.size(2), rq.size(3), values[0].size(3)), dtype=rq.dtype, device=_dev())   # :213-218
+    attn_output = hogwild_fused(query_states, cd.locations, keys, values, c.scale, frags, cd.cos, cd.sin, rotated_queries=rq,
+                                out=att_buffer)
+    out_op = torch.empty_like(attn_output)
+    rq_op = torch.empty_like(rq)
+    torch.ops.libhogatt.hogwild_fused(out_op, rq_op, c.scale, cd.locations, query_states.contiguous(), frags, keys, values, cd.cos, cd.sin)
+    torch.cuda.synchronize()
+    o_ref, _, rq_ref = oracle_fused(oracle, c)
+    assert_close("out", attn_output, o_ref, TOL["bf16"])
+    assert torch.equal(attn_output, out_op) and torch.equal(rq.view(torch.int16), rq_op.view(torch.int16))
+    assert_close("rq", rq, rq_ref, 3.2e-2)
+    flat = attn_output.transpose(1, 2).reshape(W, S, -1).contiguous()
+    assert flat.shape == (W, S, Hq * E)
+    # the two halves through the same import path
+    out2 = hogwild_sdpa(hogwild_rope(query_states, cd.cos, cd.sin), cd.locations, keys, values, c.scale)
+    torch.cuda.synchronize()
+    assert_close("sdpa out", out2, o_ref, TOL["bf16"])
