@@ -51,6 +51,8 @@ def parse_args():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (and with it the parity gate)")
     ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only: skip the other configurations under extra")
+    ap.add_argument("--variant", choices=["mfma", "valu_qk"], default="mfma",
+                    help="valu_qk = logits by VALU dot products instead of MFMA (configurations with at most 16 rows per kv head)")
     ap.add_argument("--ring-mb", type=int, default=640)
     ap.add_argument("--workload", choices=["fragments", "paged", "varlen", "stack"], default="fragments",
                     help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape; "
@@ -145,7 +147,7 @@ def make_ring(case, dev, ring_mb):
 class FragmentRun:
     """One workload configuration set up on the GPU: the ring of KV sets, one prepared hw_problem per set."""
 
-    def __init__(self, case_id, dev, args, with_rq=True):
+    def __init__(self, case_id, dev, args, with_rq=True, variant=None):
         import torch
         from inference_lib_amd import _lib, cases
         self.case = case = cases.baseline_case(case_id)
@@ -161,7 +163,8 @@ class FragmentRun:
         self.ws = None
         for keys, vals in self.ring:
             pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=keys, values=vals, scale=case.scale, out=self.out,
-                              cosines=cd.cos, sines=cd.sin, rq=self.rq, lse=self.lse, splits=args.splits)
+                              cosines=cd.cos, sines=cd.sin, rq=self.rq, lse=self.lse, splits=args.splits,
+                              variant={"mfma": 0, "valu_qk": 1}[variant or args.variant])
             if self.ws is None:
                 self.ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
             pr.set_workspace(self.ws)
@@ -263,6 +266,17 @@ def side_config(case_id, dev, args, stream):
            "step_us_p10_p90": [round(step["p10"], 3), round(step["p90"], 3)],
            "kernel_frac_of_peak": round(run.kv_bytes / kern["median"] / 1e3 / PEAK_HBM_GBS, 4),
            "step_GBps": round(run.kv_bytes / step["median"] / 1e3, 1)}
+    if run.plan.rows <= 16 and args.variant == "mfma":
+        # the matrix-core choice measured against VALU logits on the same workload (same ring, same plan)
+        del run
+        torch.cuda.empty_cache()
+        run = FragmentRun(case_id, dev, args, variant="valu_qk")
+        with torch.cuda.stream(stream):
+            for i in range(5):
+                run.step(i)
+            torch.cuda.synchronize()
+        res["valu_logits_kernel_us"] = round(time_graph(stream, run.kernel, K, **kw)["median"], 3)
+        res["valu_logits_step_us"] = round(time_graph(stream, run.step, K, **kw)["median"], 3)
     del run
     torch.cuda.empty_cache()
     return res
@@ -437,7 +451,7 @@ def main():
         del run, problems, problems_dl
         torch.cuda.empty_cache()
         cfgs = []
-        for cid in (2, 4, 5):
+        for cid in (1, 2, 4, 5):
             if cid != args.case:
                 cfgs.append(side_config(cid, dev, args, stream))
         pargs = argparse.Namespace(**vars(args))

@@ -85,7 +85,14 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
  *              spread over more workgroups that read the same KV)
+ *   variant    HW_VARIANT_MFMA (0, default): logits and output on the matrix cores.  HW_VARIANT_VALU_QK: the logits
+ *              K.Q^T by VALU dot products (v_dot2_f32_bf16 / _f16, v_fma_f32) in the same kernel, the inner product the
+ *              reference uses (src/kernels/kernel_v21.cuh:161-180); exists so that the matrix-core choice can be measured
+ *              for workloads with at most 16 query rows per kv head (hw_fused_attention, RotE == E, host lengths;
+ *              anything else returns HW_ERR_UNSUPPORTED).
  */
+#define HW_VARIANT_MFMA 0
+#define HW_VARIANT_VALU_QK 1
 typedef struct hw_problem {
     int32_t dtype;
     int32_t F, W, Hq, Hkv, S, E, Ev, RotE;
@@ -106,6 +113,7 @@ typedef struct hw_problem {
     int32_t row_blocks;
     const int32_t* cap;
     const int32_t* len_dev;
+    int32_t variant;
 } hw_problem;
 
 /* How a problem is cut into workgroups; filled by hw_plan_debug (host only, no device needed). */

@@ -43,6 +43,7 @@ class HwProblem(C.Structure):
         ("splits", C.c_int32), ("row_blocks", C.c_int32),
         ("cap", C.POINTER(C.c_int32)),
         ("len_dev", C.c_void_p),
+        ("variant", C.c_int32),
     ]
 
 
@@ -107,6 +108,7 @@ class HwAppend(C.Structure):
 
 
 HW_ROPE_EAGER, HW_ROPE_FUSED = 0, 1
+HW_VARIANT_MFMA, HW_VARIANT_VALU_QK = 0, 1
 
 
 class HogwildError(RuntimeError):
@@ -196,7 +198,8 @@ class Problem:
                  values: Sequence[torch.Tensor], scale: float, out: torch.Tensor,
                  cosines: Optional[torch.Tensor] = None, sines: Optional[torch.Tensor] = None,
                  rq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
-                 prerotated: bool = False, splits: int = 0, row_blocks: int = 0, len_dev: Optional[torch.Tensor] = None):
+                 prerotated: bool = False, splits: int = 0, row_blocks: int = 0, len_dev: Optional[torch.Tensor] = None,
+                 variant: int = 0):
         keys = [_frag3(k) for k in keys]
         values = [_frag3(v) for v in values]
         F = len(keys)
@@ -282,6 +285,7 @@ class Problem:
         p.len_dev = len_dev.data_ptr() if len_dev is not None else None
         p.splits = int(splits)
         p.row_blocks = int(row_blocks)
+        p.variant = int(variant)      # 0 = matrix cores; 1 = logits by VALU dot products (HW_VARIANT_VALU_QK, for A/B measurements)
         self.p = p
         self.prerotated = prerotated
         self._ws = None

@@ -67,6 +67,8 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     st = make_plan(p, cus, &plan, fused);
     if (st != HW_OK) return st;
     if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
+    // the VALU logits exist for what they are measured on: the fused entry with full rotary width, one row block, host lengths
+    if (p->variant == HW_VARIANT_VALU_QK && (!fused || p->RotE != p->E || plan.row_blocks != 1 || p->len_dev != nullptr)) return HW_ERR_UNSUPPORTED;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
     const void* q_in = p->q;
@@ -118,7 +120,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
 
     hipError_t e = hipSuccess;
     if (stages & HW_STAGE_ATTENTION) {
-        e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, stream);
+        e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, p->variant, stream);
         if (e != hipSuccess) return (int)e;
     }
     if (!(stages & HW_STAGE_MERGE)) return (int)e;

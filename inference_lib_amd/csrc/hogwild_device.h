@@ -46,6 +46,9 @@ template <> struct Elem<BF16> {
         f32x2 v = {a, b};
         return __builtin_bit_cast(u32, __builtin_convertvector(v, bf16x2));
     }
+    static __device__ __forceinline__ float dot(u32 a, u32 b, float c) {   // two elements per dword
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), c, false);
+    }
     static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
@@ -62,6 +65,9 @@ template <> struct Elem<F16> {
         f32x2 v = {a, b};
         return __builtin_bit_cast(u32, __builtin_convertvector(v, f16x2));
     }
+    static __device__ __forceinline__ float dot(u32 a, u32 b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+    }
     static __device__ __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     }
@@ -71,6 +77,7 @@ template <> struct Elem<F32> {
     static constexpr int size = 4;
     static __device__ __forceinline__ float to_float(store_t x) { return x; }
     static __device__ __forceinline__ store_t from_float(float f) { return f; }
+    static __device__ __forceinline__ float dot(u32 a, u32 b, float c) { return __builtin_fmaf(__uint_as_float(a), __uint_as_float(b), c); }
 };
 
 constexpr float NEG_BIG = -1.0e30f;
@@ -230,7 +237,9 @@ struct WaveState {
 };
 
 // One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
-template <class DT, int E, int EV, int RB, bool MASKED, bool QREG>
+// VS = the logits S^T = K Q^T are formed with VALU dot products (v_dot2 / v_fma) instead of MFMA, in the same lane
+// layout (row = lane % 16, eight tokens per lane): the measured alternative for workloads with few query rows.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false>
 __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
                                              WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage) {
     typedef Geo<DT, E, EV> G;
@@ -251,6 +260,26 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const
     // S^T blocks: for each 16-token block, its K operand (lane = token, 16 B of head dim per k-step) against the
     // B operand of every row block (this row's rotated query, from registers when QREG, else straight from LDS)
     f32x4 sacc[RB][2];
+    if constexpr (VS) {
+        // every lane walks the K rows of its own eight tokens (the 16 lanes of a quarter-wave read the same row: an
+        // LDS broadcast) against its row's query, 16 bytes at a time
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+            for (int idx = 0; idx < 8; ++idx) {
+                const int tok = slot_token(q, idx);
+                float acc = 0.f;
+#pragma unroll
+                for (int c = 0; c < G::CPR; ++c) {
+                    const u32x4 kk = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tok, c));
+                    const u32x4 qq = *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + c * 16);
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) acc = Elem<DT>::dot(kk[d], qq[d], acc);
+                }
+                sacc[rb][idx >> 2][idx & 3] = acc;
+            }
+        }
+    } else
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
         u32x4 kop[G::KJ];

@@ -57,7 +57,7 @@ struct MergeArgs {
     int xcd_local;      // kv head h was computed on XCD h / (Hkv/8): merge it there
 };
 
-hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream);
+hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, int variant, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& ma, int dtype, int EV, hipStream_t stream);
 hipError_t launch_rope(void* out, const void* q, const float* cosv, const float* sinv, int dtype, int F, int W, int Hq, int S,
                        int E, int RotE, hipStream_t stream);

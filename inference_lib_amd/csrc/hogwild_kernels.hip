@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "../../include/hogwild_hip.h"
 #include "hogwild_kernels.h"
 
 namespace hw {
@@ -59,9 +60,10 @@ namespace hw {
 // MINW = waves per SIMD the register budget is sized for: 2 (<= 256 VGPRs) when one 16-row block is live,
 // 1 (<= 512 VGPRs) when two row blocks or fp32 operands make the tile registers too large.
 // PF = tiles a wave keeps in flight.  PRE = queries arrive rotated (hogwild_sdpa), else fused rotation.
+// VS = logits by VALU dot products instead of MFMA (one row block only): the alternative the MFMA choice is measured against.
 // DEVLEN = the current fragment lengths come from device memory (header.len_dev); the lengths in the table are then
 // the bounds the split was planned for, and a captured launch stays valid while the segments grow up to them.
-template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE, bool DEVLEN = false>
+template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE, bool DEVLEN = false, bool VS = false>
 __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     constexpr int ROWS = RB * 16;
@@ -247,8 +249,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(c
                 const int ln = l + (PF - 1) * NWAVES;
                 load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
                 if (l < lt1 && t0 < maxlim) {
-                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
-                    else compute_tile<DT, E, EV, RB, true, QREG>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                    else compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
                 }
             }
         }
@@ -413,7 +415,17 @@ static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t 
 }
 
 template <class DT>
-static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, hipStream_t stream) {
+static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, int variant, hipStream_t stream) {
+    if (variant == HW_VARIANT_VALU_QK) {     // fused entry, one row block, lengths from the host (checked by the caller)
+        constexpr bool half = Elem<DT>::size == 2;
+        if (E == 128)
+            hipLaunchKernelGGL((attention_kernel<DT, 128, 128, 1, half ? 2 : 1, half ? 2 : 1, false, false, true>), dim3(ka.h.nwg),
+                               dim3(NTHREADS), 0, stream, ka);
+        else
+            hipLaunchKernelGGL((attention_kernel<DT, 64, 64, 1, half ? 2 : 1, half ? 2 : 1, false, false, true>), dim3(ka.h.nwg),
+                               dim3(NTHREADS), 0, stream, ka);
+        return hipGetLastError();
+    }
     if (ka.h.prerotated) {
         if (ka.h.len_dev != nullptr) return hipErrorInvalidValue;   // device-resident lengths exist for the fused entry only
         if (E == 128) return launch_attention_rb<DT, 128, 128, true, false>(ka, rb, stream);
@@ -427,11 +439,11 @@ static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, hipSt
     return launch_attention_rb<DT, 64, 64, false, false>(ka, rb, stream);
 }
 
-hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, hipStream_t stream) {
+hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, int variant, hipStream_t stream) {
     switch (dtype) {
-        case 0: return launch_attention_dt<F32>(ka, E, rb, stream);
-        case 1: return launch_attention_dt<F16>(ka, E, rb, stream);
-        default: return launch_attention_dt<BF16>(ka, E, rb, stream);
+        case 0: return launch_attention_dt<F32>(ka, E, rb, variant, stream);
+        case 1: return launch_attention_dt<F16>(ka, E, rb, variant, stream);
+        default: return launch_attention_dt<BF16>(ka, E, rb, variant, stream);
     }
 }
 

@@ -29,6 +29,7 @@ int validate(const hw_problem* p, int fused) {
     if (p == nullptr) return HW_ERR_NULL;
     if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
     if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->variant != HW_VARIANT_MFMA && p->variant != HW_VARIANT_VALU_QK) return HW_ERR_UNSUPPORTED;
     if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->E < 1 || p->Ev < 1) return HW_ERR_SHAPE;
     if (p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
     if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return HW_ERR_SHAPE;   // the row max is taken before scaling

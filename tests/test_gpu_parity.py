@@ -83,3 +83,47 @@ def test_partial_rotary(oracle, dtype, E, rot):
     assert_close("lse", lse, l_ref, TOL[dtype])
     out2, lse2, _ = run_fused(c.to(_dev()), with_rq=False)     # rotated queries go to the workspace instead
     assert torch.equal(out, out2) and torch.equal(lse, lse2)
+
+
+@pytest.mark.parametrize("idx", [1, 2])
+def test_valu_logits_variant_on_the_small_row_configs(oracle, idx):
+    """HW_VARIANT_VALU_QK (logits by v_dot2 / v_fma instead of MFMA; at most 16 rows per kv head) against the oracle on the
+    two workload configurations it is measured on, and refused where it does not exist."""
+    from inference_lib_amd import _lib, cases
+    c = cases.baseline_case(idx)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out, cosines=cd.cos,
+                      sines=cd.sin, lse=lse, variant=_lib.HW_VARIANT_VALU_QK)
+    pr.run()
+    torch.cuda.synchronize()
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL[c.dtype])
+    assert_close("lse", lse, l_ref, TOL[c.dtype])
+
+
+@pytest.mark.parametrize("dtype,E", [("bf16", 128), ("f16", 64), ("f32", 64), ("f32", 128), ("bf16", 64), ("f16", 128)])
+def test_valu_logits_variant_small(oracle, dtype, E):
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype=dtype, W=2, S=1, Hq=8, Hkv=2, E=E, lens=(100, 37, 65), seed=13)
+    cd = c.to(_dev())
+    W, Hq, S, _ = cd.q.shape
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out, cosines=cd.cos,
+                      sines=cd.sin, lse=lse, variant=_lib.HW_VARIANT_VALU_QK)
+    pr.run()
+    torch.cuda.synchronize()
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL[dtype])
+    assert_close("lse", lse, l_ref, TOL[dtype])
+    # more than 16 rows per kv head: no such kernel
+    c3 = cases.small_case(dtype=dtype, W=5, S=1, Hq=8, Hkv=2, E=E, lens=(40, 8, 8, 8, 8, 8), seed=1).to(_dev())
+    out3 = torch.empty_like(c3.q)
+    pr3 = _lib.Problem(q=c3.q, locations=c3.locations, keys=c3.keys, values=c3.values, scale=c3.scale, out=out3, cosines=c3.cos,
+                       sines=c3.sin, variant=_lib.HW_VARIANT_VALU_QK)
+    with pytest.raises(_lib.HogwildError) as ei:
+        pr3.run()
+    assert ei.value.status == -4
