@@ -53,6 +53,9 @@ def parse_args():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only: skip the other configurations under extra")
     ap.add_argument("--variant", choices=["mfma", "valu_qk"], default="mfma",
                     help="valu_qk = logits by VALU dot products instead of MFMA (configurations with at most 16 rows per kv head)")
+    ap.add_argument("--profile-steps", type=int, default=0,
+                    help="profiling mode for rocprofv3: run this many eager steps of the chosen workload over the cold ring plus the "
+                         "calibration kernels, time nothing, print a short JSON line (graphs and the other legs are skipped)")
     ap.add_argument("--ring-mb", type=int, default=640)
     ap.add_argument("--workload", choices=["fragments", "paged", "varlen", "stack"], default="fragments",
                     help="fragments = the headline fused operator; paged = hogwild_paged_sdpa decode step at the same model shape; "
@@ -282,6 +285,33 @@ def side_config(case_id, dev, args, stream):
     return res
 
 
+def profile_mode(args, dev, stream, step_fn, kv_bytes, name):
+    """What a rocprofv3 run of this script executes: eager launches only (a profiler serialises dispatches, so the
+    replay timing above would take minutes and mean nothing), the workload walking its cold ring, then the streaming
+    read and the 256 MiB copy whose known sizes scale the FETCH_SIZE / WRITE_SIZE counters."""
+    import torch
+    from inference_lib_amd import _lib
+    blib = bench_lib()
+    with torch.cuda.stream(stream):
+        for i in range(5):
+            step_fn(i)
+        torch.cuda.synchronize()
+        for i in range(args.profile_steps):
+            step_fn(5 + i)
+        torch.cuda.synchronize()
+        big = torch.empty(2 * 256 * 1024 * 1024, dtype=torch.uint8, device=dev)
+        big.random_(0, 255)
+        sink = torch.zeros(256, dtype=torch.int32, device=dev)
+        s_handle = C.c_void_p(stream.cuda_stream)
+        half = 256 * 1024 * 1024
+        for _ in range(3):
+            _lib.check(blib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), s_handle), "hw_stream_read")
+            _lib.check(blib.hw_stream_copy(big.data_ptr() + half, big.data_ptr(), half, s_handle), "hw_stream_copy")
+        torch.cuda.synchronize()
+    print(json.dumps({"profile_mode": True, "workload": name, "steps": args.profile_steps, "kv_bytes_per_step": kv_bytes,
+                      "calibration": {"stream_read_bytes": 2 * half, "stream_copy_bytes_each_way": half}}))
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -311,6 +341,10 @@ def main():
     W, Hq, S, E = cd.q.shape
     tdt = cd.q.dtype
     K, Wm = args.steps, args.warmup
+
+    if args.profile_steps > 0:
+        profile_mode(args, dev, stream, run.step, kv_bytes, f"config {args.case} ({case.name})")
+        return
 
     parity, baseline = (None, None) if args.no_cpu else cpu_leg(run, stream)
 
@@ -517,6 +551,9 @@ def bench_paged(args, dev, quick=False):
     plan = _lib.paged_plan(W=W, Hq=Hq, Hkv=Hkv, Ev=D, block_size=bs, max_blocks=nblk, num_cus=_lib.lib.hw_device_cus(), S=S,
                            splits=args.splits, total_q=(q.size(1) if varlen else None))
     K, Wm = args.steps, args.warmup
+    if getattr(args, "profile_steps", 0) > 0 and not quick:
+        profile_mode(args, dev, torch.cuda.Stream(), lambda i: problems[i % nring].run(), kv_bytes, "paged " + args.workload)
+        sys.exit(0)
     kw = dict(warmup=Wm, min_replays=10, min_total=1000) if quick else dict(warmup=Wm)
     small = dict(warmup=Wm, min_replays=10, min_total=1000)
     stream = torch.cuda.Stream()

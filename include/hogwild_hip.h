@@ -84,7 +84,8 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
- *              spread over more workgroups that read the same KV)
+ *              spread over more workgroups that read the same KV); 8 = 128-row workgroups whose waves share every K/V
+ *              tile through LDS (16-bit types without len_dev; the automatic choice beyond 64 rows per kv head)
  *   variant    HW_VARIANT_MFMA (0, default): logits and output on the matrix cores.  HW_VARIANT_VALU_QK: the logits
  *              K.Q^T by VALU dot products (v_dot2_f32_bf16 / _f16, v_fma_f32) in the same kernel, the inner product the
  *              reference uses (src/kernels/kernel_v21.cuh:161-180); exists so that the matrix-core choice can be measured
@@ -119,7 +120,7 @@ typedef struct hw_problem {
 /* How a problem is cut into workgroups; filled by hw_plan_debug (host only, no device needed). */
 typedef struct hw_plan {
     int32_t rows;             /* W*S*(Hq/Hkv): query rows that share one kv head */
-    int32_t row_blocks;       /* 16-row MFMA blocks per workgroup (1 or 2) */
+    int32_t row_blocks;       /* 16-row MFMA blocks per workgroup (1, 2 or 8) */
     int32_t row_groups;       /* workgroups along the row dimension */
     int32_t tile_tokens;      /* tokens per wave step */
     int32_t tiles_per_head;   /* sum_f ceil(len[f] / tile_tokens) */

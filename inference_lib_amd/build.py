@@ -34,7 +34,7 @@ def _run(cmd):
 
 
 def build_library() -> str:
-    srcs = [os.path.join(CSRC, n) for n in ("hogwild_kernels.hip", "hogwild_paged.hip", "hogwild_cache.hip", "hogwild_capi.hip", "hogwild_plan.cpp")]
+    srcs = [os.path.join(CSRC, n) for n in ("hogwild_kernels.hip", "hogwild_wide.hip", "hogwild_paged.hip", "hogwild_cache.hip", "hogwild_capi.hip", "hogwild_plan.cpp")]
     cmd = [HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
            "-munsafe-fp-atomics", *DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *srcs]
     _run(cmd)

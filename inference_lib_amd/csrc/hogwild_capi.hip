@@ -120,7 +120,10 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
 
     hipError_t e = hipSuccess;
     if (stages & HW_STAGE_ATTENTION) {
-        e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, p->variant, stream);
+        if (plan.row_blocks == hw::WIDE_ROW_BLOCKS)
+            e = hw::launch_attention_wide(ka, p->dtype, p->E, stream);
+        else
+            e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, p->variant, stream);
         if (e != hipSuccess) return (int)e;
     }
     if (!(stages & HW_STAGE_MERGE)) return (int)e;

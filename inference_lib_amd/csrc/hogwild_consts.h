@@ -7,6 +7,7 @@ constexpr int MAXF = 64;       // fragments per launch (table travels in the ker
 constexpr int TILE = 32;       // tokens per wave step
 constexpr int NWAVES = 4;      // waves per workgroup
 constexpr int NTHREADS = NWAVES * 64;
+constexpr int WIDE_ROW_BLOCKS = 8;   // 16-row blocks of a workgroup of the many-rows kernel (32 rows per wave)
 constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary table below)
 
 }  // namespace hw

@@ -58,6 +58,8 @@ struct MergeArgs {
 };
 
 hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, int variant, hipStream_t stream);
+// many rows per kv head: 128-row workgroups that share every K/V tile through LDS (16-bit types, host-side lengths)
+hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStream_t stream);
 hipError_t launch_merge(const MergeArgs& ma, int dtype, int EV, hipStream_t stream);
 hipError_t launch_rope(void* out, const void* q, const float* cosv, const float* sinv, int dtype, int F, int W, int Hq, int S,
                        int E, int RotE, hipStream_t stream);

@@ -70,8 +70,15 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     if ((long long)p->Hkv * ((rows_ll + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
     const int rows = (int)rows_ll;
     plan->rows = rows;
+    // up to 16 rows: one 16-row block per workgroup (two workgroups per CU); up to 64: two blocks, rows beyond 32 in a
+    // second row group that reads the same KV; more: 128-row workgroups whose four waves share every K/V tile through
+    // LDS (16-bit types, lengths known on the host) -- a CU can take in about 16 B/clk, so what counts is that every
+    // CU reads every byte once
+    const bool wide_ok = p->dtype != HW_F32 && p->len_dev == nullptr && p->variant == HW_VARIANT_MFMA;
     plan->row_blocks = rows <= 16 ? 1 : 2;
-    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
+    if (wide_ok && rows > 64) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
+    if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
+    const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rows_per_wg = 16 * plan->row_blocks;
     plan->row_groups = (rows + rows_per_wg - 1) / rows_per_wg;
     plan->tile_tokens = hw::TILE;
@@ -93,7 +100,8 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
         const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32) ? 2 : 1;
         const int target = per_cu * num_cus;
         wgs = target / (p->Hkv * plan->row_groups);
-        const int by_work = (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
+        // narrow kernels deal a workgroup's tiles to its four waves; in the wide kernel every wave takes every tile
+        const int by_work = wide ? (int)((tiles + 3) / 4) : (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
         if (wgs > by_work) wgs = by_work;
     }
     if (wgs > (int)tiles) wgs = (int)tiles;
@@ -105,7 +113,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     // rather than tiles alone: a run of tiny fragments is spread over several workgroups instead of
     // serialising their prologues in one straggler.
     {
-        const double kOpenCost = 6.0;
+        const double kOpenCost = wide ? 2.0 : 6.0;   // in tiles of the kernel's own pace (a wide workgroup takes a tile in one step)
         int nfrag_left = 0;
         for (int f = 0; f < p->F; ++f) nfrag_left += p->len[f] > 0 ? 1 : 0;
         long long tiles_left = tiles;

@@ -1,0 +1,475 @@
+// Hogwild! fragmented-KV attention for many query rows per kv head (several tokens per worker, many workers, wide GQA
+// groups): the shape where a decode step turns into a small prefill.  gfx950 (MI355X, CDNA4, wave64), 16-bit types.
+//
+// One workgroup = one kv head x one contiguous range of 32-token tiles x up to 128 query rows: each of the four
+// waves owns 32 rows (two 16-row MFMA blocks) and ALL four multiply against EVERY tile of the range.  A tile is brought
+// into LDS once per workgroup -- K and V by direct global->LDS transfers, a quarter of the tile issued by each wave --
+// and read from there by the four waves.  What bounds the narrow kernel on such shapes is the rate at which one CU can
+// take data in (about 16 B/clk through the vector memory path, whatever cache answers): with 32-row workgroups every
+// group of 32 rows streams the whole KV through its CU again, four times for 128 rows.  Here a CU takes every byte in
+// once and spreads it through LDS (each wave reads 16 KB per tile out of 128 B/clk of LDS bandwidth).
+//
+// The tiles rotate through a ring of NS LDS slots; D = NS - 2 tiles are requested ahead.  One barrier per tile: a wave
+// waits for its own transfers of tile t, all waves meet, tile t is complete in LDS; and since every wave has then left
+// tile t-1 behind, the slot of tile t-1 is free for the request issued next (tile t+D goes to slot (t+D) mod NS, which
+// is neither the slot being read nor one still in flight).  The transfers are issued from inline assembly and waited for
+// by hand (see lds_transfer).
+// Rows of different waves are different rows, so nothing is combined across waves at the end: every wave stores the
+// partial (unnormalised output, running max, sum) of its own 32 rows, and the merge kernel of the narrow path
+// (merge_kernel) finishes the job.
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "../../include/hogwild_hip.h"
+#include "hogwild_kernels.h"
+
+#ifndef HW_MARK
+#define HW_MARK(i) do { } while (0)
+#endif
+
+#include "hogwild_device.h"
+
+namespace hw {
+
+constexpr int WIDE_ROWS = 128;      // query rows per workgroup: 32 per wave
+
+// K and V slices of one kv head of a fragment as raw buffer descriptors (base, stride 0, size in bytes, flags): rows
+// beyond the fragment read as zero.  Held as plain words: the transfers below are issued from inline assembly.
+struct WideView {
+    u32x4 k, v;
+};
+__device__ __forceinline__ u32x4 raw_descriptor(unsigned long long base, unsigned bytes) {
+    u32x4 d;
+    d.x = __builtin_amdgcn_readfirstlane((u32)base);
+    d.y = __builtin_amdgcn_readfirstlane((u32)(base >> 32) & 0xffffu);
+    d.z = __builtin_amdgcn_readfirstlane(bytes);
+    d.w = 0x00020000u;
+    return d;
+}
+__device__ __forceinline__ WideView make_wide_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow) {
+    WideView w;
+    w.k = raw_descriptor(kptr + (unsigned long long)hkv * cap * krow, (unsigned)(L * krow));
+    w.v = raw_descriptor(vptr + (unsigned long long)hkv * cap * vrow, (unsigned)(L * vrow));
+    return w;
+}
+
+// One 1 KB global->LDS transfer (lane l: 16 bytes from descriptor offset `voffset` to LDS byte `lds` + 16 l), non-temporal.
+// Issued from inline assembly on purpose: the compiler waits for every transfer it knows of before a read of LDS it
+// cannot prove disjoint, which would empty the look-ahead queue at every tile; these it does not know of, and the kernel
+// waits for them itself (s_waitcnt vmcnt before the barrier of each tile).  Loads complete in order, so a compiler-
+// generated wait for one of its own loads can only become longer through them, never too short.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"   // m0 is a reserved register: it is set and used inside the one statement
+__device__ __forceinline__ void lds_transfer(const u32x4& desc, unsigned lds, unsigned voffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds" ::"s"(lds), "v"(voffset), "s"(desc) : "m0", "memory");
+}
+#pragma clang diagnostic pop
+
+// One wave's share of a tile's transfers: KPW 1 KB pieces of the K image and VPW of the V image, starting at piece
+// `first_k` / `first_v` of the slot (kslot / vslot: LDS byte addresses).  kb / vb = byte offset of the tile in the kv
+// head's slice (OOB_OFFSET for a tile that does not exist: the same number of transfers, no memory traffic, zeros in LDS).
+template <int KPW, int VPW>
+__device__ __forceinline__ void wide_request(const WideView& w, unsigned kslot, unsigned vslot, int first_k, int first_v, unsigned kb, unsigned vb,
+                                             const unsigned* koff, const unsigned* voff) {
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) lds_transfer(w.k, kslot + (first_k + j) * 1024, kb + koff[j]);
+#pragma unroll
+    for (int j = 0; j < VPW; ++j) lds_transfer(w.v, vslot + (first_v + j) * 1024, vb + voff[j]);
+}
+
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+    return __builtin_amdgcn_readfirstlane((unsigned)(size_t)HW_LDS_PTR(p));
+}
+
+// Query rotation of one fragment for the 128 rows of a workgroup (the role of QueryRotation in the narrow kernel).  The
+// rows of one (worker, token) pair share their cos/sin table row, and with 128 rows per workgroup loading it per query
+// row made the prologue the most expensive part of the kernel (a CU takes in ~16 B/clk: 64 KB of table rows against
+// 32 KB of queries).  Here the distinct table rows of the workgroup go through LDS once (first halves only: both halves
+// of the rotation read cos/sin at the first-half index, src/rope.cuh:30-46), CSMAX of them; a workgroup whose rows span
+// more (worker, token) pairs than that (GQA ratio below 4) cannot use it and takes the per-row path.
+template <class DT, int E, int QSTR>
+struct WideRotation {
+    static constexpr int SZ = Elem<DT>::size;
+    static constexpr int CH = Chunk<DT>::CH;
+    static constexpr int IPR = E / (2 * CH);                                  // chunk pairs per row
+    static constexpr int NIT = (WIDE_ROWS * IPR + NTHREADS - 1) / NTHREADS;   // chunk pairs per thread
+    static constexpr int CSMAX = 36;                                          // table rows staged per workgroup
+    static constexpr int CPW = E / 2 / 4;                                     // float4 per half table row
+    static constexpr int NCS = (CSMAX * 2 * CPW + NTHREADS - 1) / NTHREADS;   // table float4 per thread
+    static constexpr int CS_FLOATS = CSMAX * E;                               // [row][cos half | sin half]
+
+    u32x4 xa[NIT], xb[NIT];
+    f32x4 tab[NCS];
+
+    // global loads: the queries of this thread's chunk pairs and its share of the table rows ws_lo .. ws_lo + nws - 1
+    __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid, int ws_lo, int nws) {
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / IPR, slot = item % IPR;
+            const int r = (item < WIDE_ROWS * IPR && r0 + rr < a.R) ? r0 + rr : r0;
+            const RowMap rm = map_row(a, r, hkv, GQ);
+            const HW_GLOBAL char* qp = a.q + rm.qrow * E * SZ;
+            xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
+            xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + IPR) * 16);
+        }
+#pragma unroll
+        for (int k = 0; k < NCS; ++k) {
+            const int item = tid + k * NTHREADS;
+            const int wi = min(item / (2 * CPW), nws - 1), part = item % (2 * CPW);      // beyond the last row: re-read it
+            const HW_GLOBAL float* src = (part < CPW ? a.cos : a.sin) + ((size_t)f * a.W * a.S + ws_lo + wi) * E + (part % CPW) * 4;
+            tab[k] = *reinterpret_cast<const HW_GLOBAL f32x4*>(src);
+        }
+    }
+
+    // table rows into LDS (a barrier must follow before rotate())
+    __device__ __forceinline__ void stage(float* cs_lds, int tid, int nws) const {
+#pragma unroll
+        for (int k = 0; k < NCS; ++k) {
+            const int item = tid + k * NTHREADS;
+            if (item < nws * 2 * CPW) *reinterpret_cast<f32x4*>(cs_lds + item * 4) = tab[k];
+        }
+    }
+
+    __device__ __forceinline__ void rotate(const DevHeader& a, char* q_lds, const float* cs_lds, int f, int hkv, int r0, int GQ, bool write_rq,
+                                           int tid, int ws_lo) const {
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+#pragma unroll
+        for (int it = 0; it < NIT; ++it) {
+            const int item = tid + it * NTHREADS;
+            const int rr = item / IPR, slot = item % IPR;
+            if (item >= WIDE_ROWS * IPR) continue;
+            char* lrow = q_lds + rr * QSTR;
+            const bool pad = r0 + rr >= a.R;
+            const RowMap rm = map_row(a, pad ? r0 : r0 + rr, hkv, GQ);
+            const float* cs = cs_lds + (rm.ws - ws_lo) * E + slot * CH;
+            float x1[CH], x2[CH], y1[CH], y2[CH];
+            Chunk<DT>::unpack(xa[it], x1);
+            Chunk<DT>::unpack(xb[it], x2);
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const float c = cs[i], sv = cs[E / 2 + i];
+                y1[i] = x1[i] * c - x2[i] * sv;
+                y2[i] = x2[i] * c + x1[i] * sv;
+            }
+            const u32x4 z = {0, 0, 0, 0};
+            const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
+            *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : ya;
+            *reinterpret_cast<u32x4*>(lrow + (slot + IPR) * 16) = pad ? z : yb;
+            if (write_rq && !pad) {
+                HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
+                *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
+                *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + IPR) * 16) = yb;
+            }
+        }
+    }
+};
+
+template <class DT, int E, int EV, int NS, bool PRE>
+__global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const KernelArgs args) {
+    typedef Geo<DT, E, EV> G;
+    constexpr int RB = 2;                       // 16-row blocks per wave
+    constexpr int WROWS = RB * 16;              // rows per wave
+    constexpr int D = NS - 2;                   // tiles requested ahead
+    constexpr int KPW = G::KL / NWAVES;         // 1 KB K transfers each wave issues per tile
+    constexpr int VL = TILE * G::VROW / 1024;   // 1 KB V transfers per tile
+    constexpr int VPW = VL / NWAVES;
+    static_assert(G::SZ == 2 && KPW >= 1 && VPW >= 1 && D >= 1, "16-bit types, at least one transfer per wave and tile");
+
+    __shared__ __attribute__((aligned(16))) char q_lds[WIDE_ROWS * G::QSTR];
+    __shared__ int lim_lds[WIDE_ROWS];
+    typedef WideRotation<DT, E, G::QSTR> WRot;
+    __shared__ __attribute__((aligned(16))) float cs_lds[PRE ? 4 : WRot::CS_FLOATS];
+    // ring slots; K is swizzled like in the narrow kernel, V is a plain row-major image
+    struct Slot {
+        char k[G::KSTAGE];
+        char v[TILE * G::VROW];
+    };
+    struct Stub {
+        char k[16];
+        char v[16];
+    };
+    __shared__ __attribute__((aligned(16))) Slot ring0, ring1, ring2;
+    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 3), Slot, Stub>::type ring3;
+    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 4), Slot, Stub>::type ring4;
+    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 5), Slot, Stub>::type ring5;
+    static_assert(NS >= 3 && NS <= 6, "ring of three to six slots");
+    char* const kslot[6] = {ring0.k, ring1.k, ring2.k, ring3.k, ring4.k, ring5.k};
+    char* const vslot[6] = {ring0.v, ring1.v, ring2.v, ring3.v, ring4.v, ring5.v};
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int q = lane >> 4;
+
+    // the kernel arguments in one burst (see attention_kernel)
+    const int fl = lane & (MAXF - 1);
+    const unsigned long long my_k = reinterpret_cast<unsigned long long>(args.frag.k[fl]);
+    const unsigned long long my_v = reinterpret_cast<unsigned long long>(args.frag.v[fl]);
+    const FragTable::LenCap my_lc = args.frag.lc[fl];
+    const int my_len = my_lc.len;
+    const int my_cap = my_lc.cap;
+    const int my_tb = args.frag.tile_begin[fl];
+    const int my_te = args.frag.tile_begin[fl + 1];
+    int my_wt[MAX_SPLITS / 64], my_wt1[MAX_SPLITS / 64];
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        my_wt[i] = args.wg_tile[lane + 64 * i];
+        my_wt1[i] = args.wg_tile[lane + 64 * i + 1];
+    }
+    typedef int i32x16 __attribute__((ext_vector_type(16)));
+    struct HeaderBits { i32x16 lo, hi; };
+    HeaderBits hb;
+    {
+        const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(hb.lo), "=&s"(hb.hi) : "s"(argp) : "memory");
+    }
+    // this wave's share of a tile's transfers: K transfers wv*KPW .., V transfers wv*VPW ..  A transfer writes LDS
+    // linearly (lane l -> base + 16 l); the K swizzle is applied on the global side (see k_lane_offsets)
+    unsigned koff[KPW], voff[VPW];
+#pragma unroll
+    for (int j = 0; j < KPW; ++j) {
+        const int p = (wv * KPW + j) * 64 + lane;
+        const int row = p / G::CPR, slot = p % G::CPR;
+        const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+        koff[j] = row * G::KROW + ((slot ^ key) << 4);
+    }
+#pragma unroll
+    for (int j = 0; j < VPW; ++j) voff[j] = ((wv * VPW + j) * 64 + lane) * 16;
+    WaveState<RB, G::NOC> st;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        st.m[rb] = NEG_BIG;
+        st.l[rb] = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    st.fresh = true;
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");
+    const DevHeader a = __builtin_bit_cast(DevHeader, hb);
+
+    int bid = blockIdx.x;
+    if (a.xcd_remap) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
+    const int hg = fast_div(bid, a.magic_nrg);
+    const int rg = bid - hg * a.nrg;
+    const int hkv = fast_div(hg, a.magic_wg);
+    const int g = hg - hkv * a.wgs_per_head;
+    int T0 = 0, T1 = 0;
+#pragma unroll
+    for (int i = 0; i < MAX_SPLITS / 64; ++i) {
+        if ((g >> 6) == i) {
+            T0 = __builtin_amdgcn_readlane(my_wt[i], g & 63);
+            T1 = __builtin_amdgcn_readlane(my_wt1[i], g & 63);
+        }
+    }
+    const int r0 = rg * WIDE_ROWS;              // first row of the workgroup
+    const int w0 = r0 + wv * WROWS;             // first row of this wave
+    const int GQ = a.Hq / a.Hkv;
+
+    unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
+    int f = 0, L = 0, lt0 = 0, lt1 = 0;
+    bool opens_fragment = false;
+    WideView view;
+    QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE> qrot;     // pre-rotated queries, or too many (worker, token) pairs for the staged tables
+    WRot wrot;
+    // (worker, token) pairs the rows of this workgroup belong to
+    const int ws_lo = fast_div(r0, a.magic_gq);
+    const int nws = fast_div(min(r0 + WIDE_ROWS, a.R) - 1, a.magic_gq) - ws_lo + 1;
+    const bool staged = !PRE && nws <= WRot::CSMAX;          // uniform over the workgroup
+    int lm = 0;
+
+    // this wave's quarter of tile `lt` (fragment-local) into ring slot `s`; a tile that does not exist is requested out
+    // of range: the same number of transfers, no memory traffic, zeros in LDS
+    auto request = [&](int s, int lt) {
+        const bool real = lt < lt1;
+        wide_request<KPW, VPW>(view, lds_address(kslot[s]), lds_address(vslot[s]), wv * KPW, wv * VPW, real ? (unsigned)(lt * TILE * G::KROW) : OOB_OFFSET,
+                               real ? (unsigned)(lt * TILE * G::VROW) : OOB_OFFSET, koff, voff);
+    };
+
+    auto open_segment = [&]() {
+        f = __builtin_ctzll(todo);
+        todo &= todo - 1;
+        const int fb = __builtin_amdgcn_readlane(my_tb, f);
+        const int fe = __builtin_amdgcn_readlane(my_te, f);
+        const int s0 = max(T0, fb), s1 = min(T1, fe);
+        L = __builtin_amdgcn_readlane(my_len, f);
+        const unsigned long long kp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_k >> 32), f) << 32) |
+                                      (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
+        const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
+                                      (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
+        const int cap = __builtin_amdgcn_readlane(my_cap, f);
+        view = make_wide_view(kp, vp, hkv, L, cap, G::KROW, G::VROW);
+        lt0 = s0 - fb;
+        lt1 = s1 - fb;
+        opens_fragment = s0 == fb;
+        // The first tile is requested before the queries: the compiler's wait for the query loads then also waits for it
+        // (loads complete in order), which costs nothing, the tile being needed first anyway.  The other look-ahead
+        // tiles follow after the rotation, so that the rotation does not wait for them as well.
+        request(0, lt0);
+        if (!PRE && staged) wrot.load(a, f, hkv, r0, GQ, tid, ws_lo, nws);
+        else qrot.load(a, f, hkv, r0, GQ, tid);
+        // the bound of row tid / 2 (128 rows, 256 threads: two threads per row, both load; keeps the load unconditional)
+        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid >> 1), a.R - 1), a.magic_gq)];
+    };
+    bool more = todo != 0;
+    if (more) open_segment();
+
+    while (more) {
+        __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
+        if (!PRE && staged) {
+            wrot.stage(cs_lds, tid, nws);
+            __syncthreads();
+            wrot.rotate(a, q_lds, cs_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid, ws_lo);
+        } else {
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
+        }
+        if ((tid & 1) == 0) lim_lds[tid >> 1] = (r0 + (tid >> 1) < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
+        __syncthreads();
+
+        // this wave's query operands and mask bounds
+        u32x4 qreg[RB * G::KJ];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int j = 0; j < G::KJ; ++j)
+                qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * WROWS + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+        int lim[RB];
+        int maxlim = 0, minlim = 0x7fffffff;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            lim[rb] = lim_lds[wv * WROWS + rb * 16 + n];
+            const bool pad = w0 + rb * 16 + n >= a.R;
+            maxlim = max(maxlim, pad ? 0 : lim[rb]);
+            minlim = min(minlim, lim[rb]);
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
+            minlim = min(minlim, __shfl_xor(minlim, off, 64));
+        }
+        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
+        minlim = __builtin_amdgcn_readfirstlane(minlim);
+#pragma unroll
+        for (int i = 1; i < D; ++i) request(i, lt0 + i);
+
+        bool done = false;
+        for (int lt = lt0; !done; lt += NS) {
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                const int l = lt + i;
+                if (l >= lt1) {          // uniform over the workgroup: every wave leaves at the same tile
+                    done = true;
+                    break;
+                }
+                request((i + D) % NS, l + D);
+                // Wait for this wave's own transfers of tile l, then meet the other waves: tile l is complete in LDS.  The
+                // D requests issued since are the only newer memory operations that may stay outstanding (loads complete
+                // in order; stores still in flight only make the wait longer).  A plain barrier, not __syncthreads(): its
+                // release fence would wait for every outstanding transfer, the look-ahead included.
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * (KPW + VPW)) : "memory");
+                const int t0 = l * TILE;
+                if (t0 < maxlim) {
+                    TileRegs<DT, E, EV> tr;
+#pragma unroll
+                    for (int idx = 0; idx < 8; ++idx) {
+                        const char* vp = vslot[i] + slot_token(q, idx) * G::VROW + n * (G::VW * 4);   // lane n: VW dwords of the row
+                        if constexpr (G::VW == 4) {
+                            const u32x4 x = *reinterpret_cast<const u32x4*>(vp);
+                            tr.v[idx][0] = x.x;
+                            tr.v[idx][1] = x.y;
+                            tr.v[idx][2] = x.z;
+                            tr.v[idx][3] = x.w;
+                        } else {
+                            static_assert(G::VW == 2, "head dims 64 and 128");
+                            const u32x2 x = *reinterpret_cast<const u32x2*>(vp);
+                            tr.v[idx][0] = x.x;
+                            tr.v[idx][1] = x.y;
+                        }
+                    }
+                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, kslot[i]);
+                    else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, kslot[i]);
+                }
+            }
+        }
+        // the requests behind the last tile (they fetched nothing) must have landed before the ring is used again
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        more = todo != 0;
+        if (more) {
+            __syncthreads();   // every wave is done with the ring
+            open_segment();
+        }
+    }
+
+    // ---- every wave stores the partial of its own rows.  The accumulator layout scatters a row over the lanes in 16-byte
+    // pieces; written like that, a partial (17 MB per launch at 128 rows x 32 workgroups x 8 heads) would reach memory as
+    // a million partial-line writes.  So each 16-row block goes through LDS once -- the wave's own rows of q_lds, which
+    // nobody else reads and the wave itself no longer needs -- and leaves as whole 512-byte rows, 1 KB per store. ----
+    {
+        constexpr int OSTR = EV + 4;                                  // floats per staged row (padded against bank conflicts)
+        static_assert(16 * OSTR * 4 <= WROWS * G::QSTR, "a 16-row block fits into the wave's rows of q_lds");
+        float* stage = reinterpret_cast<float*>(q_lds + wv * WROWS * G::QSTR);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const float lsum = quarter_sum(st.l[rb]);
+            const int row0 = w0 + rb * 16;                            // first row of the block
+            const size_t prow0 = (size_t)(hkv * a.wgs_per_head + g) * a.R + row0;
+#pragma unroll
+            for (int c0 = 0; c0 < G::NOC; c0 += 4)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    *reinterpret_cast<f32x4*>(stage + n * OSTR + out_ev<DT, EV>(c0, 4 * q + i)) =
+                        f32x4{st.o[rb][c0][i], st.o[rb][c0 + 1][i], st.o[rb][c0 + 2][i], st.o[rb][c0 + 3][i]};
+            if (q == 0 && row0 + n < a.R) *reinterpret_cast<HW_GLOBAL f32x2*>(a.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
+            // (one wave: the LDS writes above are complete before the reads below are issued, in program order)
+            const int nvalid = min(16, a.R - row0);                   // rows of the block that exist
+            HW_GLOBAL float* dst = a.part_o + prow0 * EV;
+#pragma unroll
+            for (int ps = 0; ps < 16 * EV / 256; ++ps) {              // 64 lanes x 4 floats per pass
+                const int idx = ps * 256 + lane * 4;
+                const int rr = idx / EV, e = idx % EV;
+                if (rr < nvalid) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * OSTR + e);
+            }
+        }
+    }
+
+    // rotated queries of zero-length fragments are still part of the operator's visible output
+    if (!PRE && a.rq != nullptr && g == 0) {
+        unsigned long long empty = __ballot(lane < a.F && my_len == 0);
+        while (empty != 0) {
+            f = __builtin_ctzll(empty);
+            empty &= empty - 1;
+            __syncthreads();
+            QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE> qempty;
+            qempty.load(a, f, hkv, r0, GQ, tid);
+            qempty.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
+        }
+    }
+}
+
+template <class DT>
+static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
+    constexpr int NS = 5;
+    if (ka.h.prerotated) {
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+    } else {
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, false>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, false>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStream_t stream) {
+    if (ka.h.len_dev != nullptr) return hipErrorInvalidValue;
+    switch (dtype) {
+        case 1: return launch_wide_dt<F16>(ka, E, stream);
+        case 2: return launch_wide_dt<BF16>(ka, E, stream);
+        default: return hipErrorInvalidValue;     // 16-bit types only
+    }
+}
+
+}  // namespace hw

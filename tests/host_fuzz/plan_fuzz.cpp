@@ -73,7 +73,7 @@ static void fuzz_fragments(std::mt19937_64& rng) {
     for (int f = p.F; f <= HW_MAX_FRAGMENTS; ++f) CHECK(plan.tile_begin[f] == tiles, "tile_begin tail %d", f);
     const int rows = p.W * p.S * (p.Hq / p.Hkv);
     CHECK(plan.rows == rows && plan.tiles_per_head == tiles, "rows / tiles");
-    CHECK(plan.row_blocks == 1 || plan.row_blocks == 2, "row_blocks %d", plan.row_blocks);
+    CHECK(plan.row_blocks == 1 || plan.row_blocks == 2 || plan.row_blocks == 8, "row_blocks %d", plan.row_blocks);
     CHECK((long long)plan.row_groups * 16 * plan.row_blocks >= rows && (long long)(plan.row_groups - 1) * 16 * plan.row_blocks < rows, "row groups");
     const int wgs = plan.wgs_per_head;
     CHECK(wgs >= 1 && wgs <= HW_MAX_SPLITS, "wgs %d", wgs);

@@ -235,3 +235,64 @@ def test_graph_replay_matches_eager():
         pe.run()
         torch.cuda.synchronize()
         assert torch.equal(out_g, out_e), f"replay {it} differs from the eager launch"
+
+
+# ------------------------------------------------------------------------------------------------ many rows per kv head
+@pytest.mark.parametrize("dtype,E,W,S,Hq,Hkv,lens", [
+    ("f16", 128, 4, 4, 16, 2, (300, 64, 33, 70, 129)),        # 128 rows per kv head: one full row group
+    ("bf16", 128, 3, 3, 14, 2, (257, 31, 0, 64)),             # 63 rows forced into the wide kernel, an empty fragment
+    ("bf16", 64, 5, 4, 16, 2, (200, 40, 41, 42, 43, 44)),     # 160 rows: two row groups, the second partly filled
+    ("f16", 64, 9, 2, 6, 2, (90, 10, 20, 30, 40, 50, 60, 70, 80, 33)),   # GQA 3: more (worker, token) pairs than staged table rows
+    ("bf16", 128, 2, 40, 8, 2, (500, 100, 120)),              # 40 query tokens per worker (prefill-like), 320 rows
+])
+def test_wide_kernel_against_oracle(oracle, dtype, E, W, S, Hq, Hkv, lens):
+    """The 128-row workgroups (row_blocks = 8; chosen automatically beyond 64 rows per kv head) against the oracle, and
+    bit-identical to nothing: the narrow kernel sums in another order, so both are compared with the oracle."""
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype=dtype, W=W, S=S, Hq=Hq, Hkv=Hkv, E=E, lens=lens, seed=len(lens) + W)
+    cd = c.to(_dev())
+    rows = W * S * (Hq // Hkv)
+    print(f"wide case {c.name}: {rows} rows per kv head, lens {lens}", flush=True)
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    for rb in (8, 2):
+        out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+        rq = torch.full((c.F, W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out, cosines=cd.cos,
+                          sines=cd.sin, rq=rq, lse=lse, row_blocks=rb)
+        pr.run()
+        torch.cuda.synchronize()
+        assert_close(f"out rb={rb}", out, o_ref, TOL[dtype])
+        assert_close(f"lse rb={rb}", lse, l_ref, TOL[dtype])
+        assert_close(f"rq rb={rb}", rq, rq_ref, 3.2e-2)
+    # pre-rotated queries through the same kernel
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    pr = _lib.Problem(q=rq, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out, prerotated=True, row_blocks=8)
+    pr.run()
+    torch.cuda.synchronize()
+    o2, _ = oracle.sdpa_fragments(np64(rq), c.locations.numpy(), [np64(k) for k in c.keys], [np64(v) for v in c.values], c.scale)
+    assert_close("sdpa out", out, o2, TOL[dtype])
+
+
+def test_wide_kernel_split_invariance_and_refusals():
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype="bf16", W=4, S=4, Hq=16, Hkv=2, E=128, lens=(700, 64, 33, 70, 129), seed=4)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    outs = []
+    for splits in (0, 1, 3, 7):
+        out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out, cosines=cd.cos,
+                          sines=cd.sin, row_blocks=8, splits=splits)
+        pr.run()
+        torch.cuda.synchronize()
+        outs.append(out.float())
+    for o in outs[1:]:
+        assert (o - outs[0]).abs().max().item() <= 2.0 ** -7 * outs[0].abs().max().item() + 1e-3
+    # fp32 has no such kernel: the request is ignored (the narrow kernel runs), never a wrong launch
+    c32 = cases.small_case(dtype="f32", W=4, S=4, Hq=16, Hkv=2, E=64, lens=(100, 20, 21, 22, 23), seed=2).to(_dev())
+    out32 = torch.full(c32.q.shape, float("nan"), dtype=torch.float32, device=_dev())
+    _lib.Problem(q=c32.q, locations=c32.locations, keys=c32.keys, values=c32.values, scale=c32.scale, out=out32, cosines=c32.cos,
+                 sines=c32.sin, row_blocks=8).run()
+    torch.cuda.synchronize()
+    assert torch.isfinite(out32).all()
