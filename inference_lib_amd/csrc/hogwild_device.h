@@ -227,6 +227,29 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
     }
 }
 
+// The V rows of a tile that lies complete in LDS, row-major (VROW bytes per token), in the layout of TileRegs (the
+// kernel whose waves share every tile).
+template <class DT, int E, int EV>
+__device__ __forceinline__ void read_v_rows(const char* vimg, int n, int q, TileRegs<DT, E, EV>& t) {
+    typedef Geo<DT, E, EV> G;
+#pragma unroll
+    for (int idx = 0; idx < 8; ++idx) {
+        const char* vp = vimg + slot_token(q, idx) * G::VROW + n * (G::VW * 4);   // lane n: VW dwords of the row
+        if constexpr (G::VW == 4) {
+            const u32x4 x = *reinterpret_cast<const u32x4*>(vp);
+            t.v[idx][0] = x.x;
+            t.v[idx][1] = x.y;
+            t.v[idx][2] = x.z;
+            t.v[idx][3] = x.w;
+        } else {
+            static_assert(G::VW == 2, "head dims 64 and 128");
+            const u32x2 x = *reinterpret_cast<const u32x2*>(vp);
+            t.v[idx][0] = x.x;
+            t.v[idx][1] = x.y;
+        }
+    }
+}
+
 // Running state of one wave: RB row blocks of 16 rows each.
 template <int RB, int NOC>
 struct WaveState {
@@ -584,12 +607,12 @@ __device__ __forceinline__ RowMap map_row(const DevHeader& a, int r, int hkv, in
 // item count per thread is a compile-time constant.  Index convention of src/rope.cuh:18-51: both halves
 // read cos/sin at the first-half index.
 // PRE = the queries arrive already rotated, [F,W,Hq,S,E] (the hogwild_sdpa entry): one item = one chunk copy.
-template <class DT, int E, int ROWS, int QSTR, bool PRE>
+template <class DT, int E, int ROWS, int QSTR, bool PRE, int NT = NTHREADS>
 struct QueryRotation {
     static constexpr int SZ = Elem<DT>::size;
     static constexpr int CH = Chunk<DT>::CH;
     static constexpr int IPR = PRE ? E / CH : E / (2 * CH);                  // items per row
-    static constexpr int NIT = (ROWS * IPR + NTHREADS - 1) / NTHREADS;       // items per thread
+    static constexpr int NIT = (ROWS * IPR + NT - 1) / NT;       // items per thread
 
     u32x4 xa[NIT];
     u32x4 xb[PRE ? 1 : NIT];
@@ -599,7 +622,7 @@ struct QueryRotation {
         const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
-            const int item = tid + it * NTHREADS;
+            const int item = tid + it * NT;
             const int rr = item / IPR, slot = item % IPR;
             // rows beyond R (MFMA padding) and threads beyond the item count read row 0: harmless, and keeps the
             // loads out of divergent control flow
@@ -624,7 +647,7 @@ struct QueryRotation {
         const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
-            const int item = tid + it * NTHREADS;
+            const int item = tid + it * NT;
             const int rr = item / IPR, slot = item % IPR;
             if (item >= ROWS * IPR) continue;
             char* lrow = q_lds + rr * QSTR;

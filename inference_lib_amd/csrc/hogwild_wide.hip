@@ -3,8 +3,8 @@
 //
 // One workgroup = one kv head x one contiguous range of 32-token tiles x up to 128 query rows: each of the four
 // waves owns 32 rows (two 16-row MFMA blocks) and ALL four multiply against EVERY tile of the range.  A tile is brought
-// into LDS once per workgroup -- K and V by direct global->LDS transfers, a quarter of the tile issued by each wave --
-// and read from there by the four waves.  What bounds the narrow kernel on such shapes is the rate at which one CU can
+// into LDS once per workgroup -- K and V by direct global->LDS transfers, the K image issued by the first half of the
+// waves and the V image by the second -- and read from there by all of them.  What bounds the narrow kernel on such shapes is the rate at which one CU can
 // take data in (about 16 B/clk through the vector memory path, whatever cache answers): with 32-row workgroups every
 // group of 32 rows streams the whole KV through its CU again, four times for 128 rows.  Here a CU takes every byte in
 // once and spreads it through LDS (each wave reads 16 KB per tile out of 128 B/clk of LDS bandwidth).
@@ -26,21 +26,15 @@
 #include "../../include/hogwild_hip.h"
 #include "hogwild_kernels.h"
 
-#ifndef HW_MARK
-#define HW_MARK(i) do { } while (0)
-#endif
-
 #include "hogwild_device.h"
 
 namespace hw {
 
+
 constexpr int WIDE_ROWS = 128;      // query rows per workgroup: 32 per wave
 
-// K and V slices of one kv head of a fragment as raw buffer descriptors (base, stride 0, size in bytes, flags): rows
-// beyond the fragment read as zero.  Held as plain words: the transfers below are issued from inline assembly.
-struct WideView {
-    u32x4 k, v;
-};
+// A slice of device memory as a raw buffer descriptor (base, stride 0, size in bytes, flags): reads beyond the size
+// return zero.  Held as plain words: the transfers below are issued from inline assembly.
 __device__ __forceinline__ u32x4 raw_descriptor(unsigned long long base, unsigned bytes) {
     u32x4 d;
     d.x = __builtin_amdgcn_readfirstlane((u32)base);
@@ -49,13 +43,6 @@ __device__ __forceinline__ u32x4 raw_descriptor(unsigned long long base, unsigne
     d.w = 0x00020000u;
     return d;
 }
-__device__ __forceinline__ WideView make_wide_view(unsigned long long kptr, unsigned long long vptr, int hkv, int L, int cap, int krow, int vrow) {
-    WideView w;
-    w.k = raw_descriptor(kptr + (unsigned long long)hkv * cap * krow, (unsigned)(L * krow));
-    w.v = raw_descriptor(vptr + (unsigned long long)hkv * cap * vrow, (unsigned)(L * vrow));
-    return w;
-}
-
 // One 1 KB global->LDS transfer (lane l: 16 bytes from descriptor offset `voffset` to LDS byte `lds` + 16 l), non-temporal.
 // Issued from inline assembly on purpose: the compiler waits for every transfer it knows of before a read of LDS it
 // cannot prove disjoint, which would empty the look-ahead queue at every tile; these it does not know of, and the kernel
@@ -68,16 +55,13 @@ __device__ __forceinline__ void lds_transfer(const u32x4& desc, unsigned lds, un
 }
 #pragma clang diagnostic pop
 
-// One wave's share of a tile's transfers: KPW 1 KB pieces of the K image and VPW of the V image, starting at piece
-// `first_k` / `first_v` of the slot (kslot / vslot: LDS byte addresses).  kb / vb = byte offset of the tile in the kv
-// head's slice (OOB_OFFSET for a tile that does not exist: the same number of transfers, no memory traffic, zeros in LDS).
-template <int KPW, int VPW>
-__device__ __forceinline__ void wide_request(const WideView& w, unsigned kslot, unsigned vslot, int first_k, int first_v, unsigned kb, unsigned vb,
-                                             const unsigned* koff, const unsigned* voff) {
+// One wave's share of a tile's transfers: TPW 1 KB pieces of ONE image (the first half of the waves fill K, the second
+// half V), into LDS bytes `slot` + 1024 j.  `tile` = byte offset of the tile in the kv head's slice (OOB_OFFSET for a
+// tile that does not exist: the same number of transfers, no memory traffic, zeros in LDS).
+template <int TPW>
+__device__ __forceinline__ void wide_request(const u32x4& desc, unsigned slot, unsigned tile, const unsigned* off) {
 #pragma unroll
-    for (int j = 0; j < KPW; ++j) lds_transfer(w.k, kslot + (first_k + j) * 1024, kb + koff[j]);
-#pragma unroll
-    for (int j = 0; j < VPW; ++j) lds_transfer(w.v, vslot + (first_v + j) * 1024, vb + voff[j]);
+    for (int j = 0; j < TPW; ++j) lds_transfer(desc, slot + j * 1024, tile + off[j]);
 }
 
 __device__ __forceinline__ unsigned lds_address(const void* p) {
@@ -90,15 +74,15 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
 // 32 KB of queries).  Here the distinct table rows of the workgroup go through LDS once (first halves only: both halves
 // of the rotation read cos/sin at the first-half index, src/rope.cuh:30-46), CSMAX of them; a workgroup whose rows span
 // more (worker, token) pairs than that (GQA ratio below 4) cannot use it and takes the per-row path.
-template <class DT, int E, int QSTR>
+template <class DT, int E, int QSTR, int NT>
 struct WideRotation {
     static constexpr int SZ = Elem<DT>::size;
     static constexpr int CH = Chunk<DT>::CH;
     static constexpr int IPR = E / (2 * CH);                                  // chunk pairs per row
-    static constexpr int NIT = (WIDE_ROWS * IPR + NTHREADS - 1) / NTHREADS;   // chunk pairs per thread
+    static constexpr int NIT = (WIDE_ROWS * IPR + NT - 1) / NT;   // chunk pairs per thread
     static constexpr int CSMAX = 36;                                          // table rows staged per workgroup
     static constexpr int CPW = E / 2 / 4;                                     // float4 per half table row
-    static constexpr int NCS = (CSMAX * 2 * CPW + NTHREADS - 1) / NTHREADS;   // table float4 per thread
+    static constexpr int NCS = (CSMAX * 2 * CPW + NT - 1) / NT;   // table float4 per thread
     static constexpr int CS_FLOATS = CSMAX * E;                               // [row][cos half | sin half]
 
     u32x4 xa[NIT], xb[NIT];
@@ -108,7 +92,7 @@ struct WideRotation {
     __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid, int ws_lo, int nws) {
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
-            const int item = tid + it * NTHREADS;
+            const int item = tid + it * NT;
             const int rr = item / IPR, slot = item % IPR;
             const int r = (item < WIDE_ROWS * IPR && r0 + rr < a.R) ? r0 + rr : r0;
             const RowMap rm = map_row(a, r, hkv, GQ);
@@ -118,7 +102,7 @@ struct WideRotation {
         }
 #pragma unroll
         for (int k = 0; k < NCS; ++k) {
-            const int item = tid + k * NTHREADS;
+            const int item = tid + k * NT;
             const int wi = min(item / (2 * CPW), nws - 1), part = item % (2 * CPW);      // beyond the last row: re-read it
             const HW_GLOBAL float* src = (part < CPW ? a.cos : a.sin) + ((size_t)f * a.W * a.S + ws_lo + wi) * E + (part % CPW) * 4;
             tab[k] = *reinterpret_cast<const HW_GLOBAL f32x4*>(src);
@@ -129,7 +113,7 @@ struct WideRotation {
     __device__ __forceinline__ void stage(float* cs_lds, int tid, int nws) const {
 #pragma unroll
         for (int k = 0; k < NCS; ++k) {
-            const int item = tid + k * NTHREADS;
+            const int item = tid + k * NT;
             if (item < nws * 2 * CPW) *reinterpret_cast<f32x4*>(cs_lds + item * 4) = tab[k];
         }
     }
@@ -139,7 +123,7 @@ struct WideRotation {
         const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
-            const int item = tid + it * NTHREADS;
+            const int item = tid + it * NT;
             const int rr = item / IPR, slot = item % IPR;
             if (item >= WIDE_ROWS * IPR) continue;
             char* lrow = q_lds + rr * QSTR;
@@ -168,37 +152,27 @@ struct WideRotation {
     }
 };
 
-template <class DT, int E, int EV, int NS, bool PRE>
-__global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const KernelArgs args) {
+template <class DT, int E, int EV, int NS, bool PRE, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
-    constexpr int RB = 2;                       // 16-row blocks per wave
+    constexpr int NT = NW * 64;                 // threads per workgroup
+    constexpr int RB = WIDE_ROWS / 16 / NW;     // 16-row blocks per wave
     constexpr int WROWS = RB * 16;              // rows per wave
+    constexpr int TPR = NT / WIDE_ROWS;         // threads per row where a row is handled by a group of threads
     constexpr int D = NS - 2;                   // tiles requested ahead
-    constexpr int KPW = G::KL / NWAVES;         // 1 KB K transfers each wave issues per tile
-    constexpr int VL = TILE * G::VROW / 1024;   // 1 KB V transfers per tile
-    constexpr int VPW = VL / NWAVES;
-    static_assert(G::SZ == 2 && KPW >= 1 && VPW >= 1 && D >= 1, "16-bit types, at least one transfer per wave and tile");
+    constexpr int KBYTES = G::KSTAGE;           // K image of a tile in LDS
+    constexpr int VBYTES = TILE * G::VROW;      // V image
+    constexpr int TPW = (KBYTES + VBYTES) / 1024 / NW;   // 1 KB transfers each wave issues per tile
+    constexpr int SLOT = KBYTES + VBYTES;
+    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && D >= 1 && RB >= 1 && NS >= 3,
+                  "16-bit types; a wave's transfers belong to one image");
 
     __shared__ __attribute__((aligned(16))) char q_lds[WIDE_ROWS * G::QSTR];
     __shared__ int lim_lds[WIDE_ROWS];
-    typedef WideRotation<DT, E, G::QSTR> WRot;
+    typedef WideRotation<DT, E, G::QSTR, NT> WRot;
     __shared__ __attribute__((aligned(16))) float cs_lds[PRE ? 4 : WRot::CS_FLOATS];
-    // ring slots; K is swizzled like in the narrow kernel, V is a plain row-major image
-    struct Slot {
-        char k[G::KSTAGE];
-        char v[TILE * G::VROW];
-    };
-    struct Stub {
-        char k[16];
-        char v[16];
-    };
-    __shared__ __attribute__((aligned(16))) Slot ring0, ring1, ring2;
-    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 3), Slot, Stub>::type ring3;
-    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 4), Slot, Stub>::type ring4;
-    __shared__ __attribute__((aligned(16))) typename std::conditional<(NS > 5), Slot, Stub>::type ring5;
-    static_assert(NS >= 3 && NS <= 6, "ring of three to six slots");
-    char* const kslot[6] = {ring0.k, ring1.k, ring2.k, ring3.k, ring4.k, ring5.k};
-    char* const vslot[6] = {ring0.v, ring1.v, ring2.v, ring3.v, ring4.v, ring5.v};
+    // ring slots: [K image | V image]; K is swizzled like in the narrow kernel, V is a plain row-major image
+    __shared__ __attribute__((aligned(16))) char ring[NS * SLOT];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -228,18 +202,21 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
         const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
         asm volatile("s_load_dwordx16 %0, %2, 0x0\n\ts_load_dwordx16 %1, %2, 0x40" : "=&s"(hb.lo), "=&s"(hb.hi) : "s"(argp) : "memory");
     }
-    // this wave's share of a tile's transfers: K transfers wv*KPW .., V transfers wv*VPW ..  A transfer writes LDS
-    // linearly (lane l -> base + 16 l); the K swizzle is applied on the global side (see k_lane_offsets)
-    unsigned koff[KPW], voff[VPW];
+    // this wave's share of a tile's transfers.  A transfer writes LDS linearly (lane l -> base + 16 l); the K swizzle is
+    // applied on the global side (see k_lane_offsets)
+    const bool k_wave = wv < NW / 2;
+    const int first = (k_wave ? wv : wv - NW / 2) * TPW;          // first 1 KB piece of the image
+    unsigned off[TPW];
 #pragma unroll
-    for (int j = 0; j < KPW; ++j) {
-        const int p = (wv * KPW + j) * 64 + lane;
+    for (int j = 0; j < TPW; ++j) {
+        const int p = (first + j) * 64 + lane;
         const int row = p / G::CPR, slot = p % G::CPR;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
-        koff[j] = row * G::KROW + ((slot ^ key) << 4);
+        off[j] = k_wave ? row * G::KROW + ((slot ^ key) << 4) : p * 16;
     }
-#pragma unroll
-    for (int j = 0; j < VPW; ++j) voff[j] = ((wv * VPW + j) * 64 + lane) * 16;
+    const unsigned long long my_image_ptr = k_wave ? my_k : my_v;   // lane f: this wave's image of fragment f
+    const int image_row = k_wave ? G::KROW : G::VROW;               // bytes per token in it
+    const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;   // in slot 0
     WaveState<RB, G::NOC> st;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -273,8 +250,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
     unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
     int f = 0, L = 0, lt0 = 0, lt1 = 0;
     bool opens_fragment = false;
-    WideView view;
-    QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE> qrot;     // pre-rotated queries, or too many (worker, token) pairs for the staged tables
+    u32x4 view = {0, 0, 0, 0};                               // this wave's image of the current fragment (K or V slice)
+    QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE, NT> qrot;     // pre-rotated queries, or too many (worker, token) pairs for the staged tables
     WRot wrot;
     // (worker, token) pairs the rows of this workgroup belong to
     const int ws_lo = fast_div(r0, a.magic_gq);
@@ -282,12 +259,11 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
     const bool staged = !PRE && nws <= WRot::CSMAX;          // uniform over the workgroup
     int lm = 0;
 
-    // this wave's quarter of tile `lt` (fragment-local) into ring slot `s`; a tile that does not exist is requested out
-    // of range: the same number of transfers, no memory traffic, zeros in LDS
-    auto request = [&](int s, int lt) {
-        const bool real = lt < lt1;
-        wide_request<KPW, VPW>(view, lds_address(kslot[s]), lds_address(vslot[s]), wv * KPW, wv * VPW, real ? (unsigned)(lt * TILE * G::KROW) : OOB_OFFSET,
-                               real ? (unsigned)(lt * TILE * G::VROW) : OOB_OFFSET, koff, voff);
+    // this wave's share of tile `lt` (fragment-local) into ring slot `sl`; a tile that does not exist is requested out of
+    // range: the same number of transfers, no memory traffic, zeros in LDS
+    auto request = [&](int sl, int lt) {
+        const unsigned tile_bytes = (unsigned)(lt * TILE * image_row);
+        wide_request<TPW>(view, my_image + sl * SLOT, lt < lt1 ? tile_bytes : OOB_OFFSET, off);
     };
 
     auto open_segment = [&]() {
@@ -297,12 +273,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
         const int fe = __builtin_amdgcn_readlane(my_te, f);
         const int s0 = max(T0, fb), s1 = min(T1, fe);
         L = __builtin_amdgcn_readlane(my_len, f);
-        const unsigned long long kp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_k >> 32), f) << 32) |
-                                      (unsigned)__builtin_amdgcn_readlane((int)my_k, f);
-        const unsigned long long vp = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_v >> 32), f) << 32) |
-                                      (unsigned)__builtin_amdgcn_readlane((int)my_v, f);
+        const unsigned long long base = ((unsigned long long)(unsigned)__builtin_amdgcn_readlane((int)(my_image_ptr >> 32), f) << 32) |
+                                        (unsigned)__builtin_amdgcn_readlane((int)my_image_ptr, f);
         const int cap = __builtin_amdgcn_readlane(my_cap, f);
-        view = make_wide_view(kp, vp, hkv, L, cap, G::KROW, G::VROW);
+        view = raw_descriptor(base + (unsigned long long)hkv * cap * image_row, (unsigned)(L * image_row));
         lt0 = s0 - fb;
         lt1 = s1 - fb;
         opens_fragment = s0 == fb;
@@ -312,8 +286,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
         request(0, lt0);
         if (!PRE && staged) wrot.load(a, f, hkv, r0, GQ, tid, ws_lo, nws);
         else qrot.load(a, f, hkv, r0, GQ, tid);
-        // the bound of row tid / 2 (128 rows, 256 threads: two threads per row, both load; keeps the load unconditional)
-        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid >> 1), a.R - 1), a.magic_gq)];
+        // the bound of row tid / TPR (TPR threads per row, all load: keeps the load unconditional)
+        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + tid / TPR, a.R - 1), a.magic_gq)];
     };
     bool more = todo != 0;
     if (more) open_segment();
@@ -327,8 +301,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
         } else {
             qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
         }
-        if ((tid & 1) == 0) lim_lds[tid >> 1] = (r0 + (tid >> 1) < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
-        __syncthreads();
+        if (tid % TPR == 0) lim_lds[tid / TPR] = (r0 + tid / TPR < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
+        // q_lds and lim_lds become visible: a barrier for LDS only.  __syncthreads() would also wait for the stores of
+        // the rotated queries to be acknowledged by memory, which nobody here depends on.
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
         // this wave's query operands and mask bounds
         u32x4 qreg[RB * G::KJ];
@@ -370,28 +346,14 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
                 // D requests issued since are the only newer memory operations that may stay outstanding (loads complete
                 // in order; stores still in flight only make the wait longer).  A plain barrier, not __syncthreads(): its
                 // release fence would wait for every outstanding transfer, the look-ahead included.
-                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * (KPW + VPW)) : "memory");
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
                 const int t0 = l * TILE;
                 if (t0 < maxlim) {
+                    const char* slot = ring + i * SLOT;
                     TileRegs<DT, E, EV> tr;
-#pragma unroll
-                    for (int idx = 0; idx < 8; ++idx) {
-                        const char* vp = vslot[i] + slot_token(q, idx) * G::VROW + n * (G::VW * 4);   // lane n: VW dwords of the row
-                        if constexpr (G::VW == 4) {
-                            const u32x4 x = *reinterpret_cast<const u32x4*>(vp);
-                            tr.v[idx][0] = x.x;
-                            tr.v[idx][1] = x.y;
-                            tr.v[idx][2] = x.z;
-                            tr.v[idx][3] = x.w;
-                        } else {
-                            static_assert(G::VW == 2, "head dims 64 and 128");
-                            const u32x2 x = *reinterpret_cast<const u32x2*>(vp);
-                            tr.v[idx][0] = x.x;
-                            tr.v[idx][1] = x.y;
-                        }
-                    }
-                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, kslot[i]);
-                    else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, kslot[i]);
+                    read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
+                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, slot);
+                    else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, slot);
                 }
             }
         }
@@ -406,12 +368,13 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
 
     // ---- every wave stores the partial of its own rows.  The accumulator layout scatters a row over the lanes in 16-byte
     // pieces; written like that, a partial (17 MB per launch at 128 rows x 32 workgroups x 8 heads) would reach memory as
-    // a million partial-line writes.  So each 16-row block goes through LDS once -- the wave's own rows of q_lds, which
-    // nobody else reads and the wave itself no longer needs -- and leaves as whole 512-byte rows, 1 KB per store. ----
+    // a million partial-line writes.  So each 16-row block goes through LDS once -- a piece of the ring, which no tile
+    // needs any more -- and leaves as whole rows, 1 KB per store. ----
     {
         constexpr int OSTR = EV + 4;                                  // floats per staged row (padded against bank conflicts)
-        static_assert(16 * OSTR * 4 <= WROWS * G::QSTR, "a 16-row block fits into the wave's rows of q_lds");
-        float* stage = reinterpret_cast<float*>(q_lds + wv * WROWS * G::QSTR);
+        static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+        __syncthreads();                                              // every wave has left the last tile
+        float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
             const float lsum = quarter_sum(st.l[rb]);
@@ -424,7 +387,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
                     *reinterpret_cast<f32x4*>(stage + n * OSTR + out_ev<DT, EV>(c0, 4 * q + i)) =
                         f32x4{st.o[rb][c0][i], st.o[rb][c0 + 1][i], st.o[rb][c0 + 2][i], st.o[rb][c0 + 3][i]};
             if (q == 0 && row0 + n < a.R) *reinterpret_cast<HW_GLOBAL f32x2*>(a.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
-            // (one wave: the LDS writes above are complete before the reads below are issued, in program order)
+            // (one wave: the LDS writes above are complete before the reads below are issued, in program order, and
+            // the reads before the next block's writes)
             const int nvalid = min(16, a.R - row0);                   // rows of the block that exist
             HW_GLOBAL float* dst = a.part_o + prow0 * EV;
 #pragma unroll
@@ -443,22 +407,30 @@ __global__ __launch_bounds__(NTHREADS, 1) void attention_wide_kernel(const Kerne
             f = __builtin_ctzll(empty);
             empty &= empty - 1;
             __syncthreads();
-            QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE> qempty;
+            QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE, NT> qempty;
             qempty.load(a, f, hkv, r0, GQ, tid);
             qempty.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
         }
     }
 }
 
+// Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
+// usual cure for a loop that waits) double what the waves read out of LDS per tile, and the kernel got slower by a
+// tenth (27.3 against 24.7 us at 128 rows x 16 K tokens x 8 kv heads, fp16).
+#ifndef HW_WIDE_WAVES
+#define HW_WIDE_WAVES 4
+#endif
+
 template <class DT>
 static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
     constexpr int NS = 5;
+    constexpr int NW = HW_WIDE_WAVES;
     if (ka.h.prerotated) {
-        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
-        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
     } else {
-        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, false>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
-        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, false>), dim3(ka.h.nwg), dim3(NTHREADS), 0, stream, ka);
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, false, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, false, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
     }
     return hipGetLastError();
 }
