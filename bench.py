@@ -451,7 +451,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / PEAK_HBM_GBS, 4),
             "traffic": load_traffic(f"attention_kernel/{case.name}"),
-            "kernel": "hw::attention_kernel",
+            "kernel": "hw::attention_wide_kernel" if run.plan.row_blocks == 8 else "hw::attention_kernel",
             "kernel_us_avg": round(kern["median"], 3),
             "kernel_us_p10_p90": [round(kern["p10"], 3), round(kern["p90"], 3)],
             "timing": f"HIP event pairs around each of {kern['replays']} back-to-back replays of a graph of K attention-kernel launches "
