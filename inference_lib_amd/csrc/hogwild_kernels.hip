@@ -1,7 +1,8 @@
 // Hogwild! fragmented-KV decode attention for gfx950 (MI355X, CDNA4, wave64).
 //
 // One workgroup = one kv head x one contiguous range of 32-token tiles (crossing fragment boundaries)
-// x up to 32 query rows, where a "row" is one (worker, token, q-head-in-group) triple.  All rows that
+// x up to 32 query rows, where a "row" is one (worker, token, q-head-in-group) triple (more than 64 rows per
+// kv head: attention_wide_kernel, hogwild_wide.hip).  All rows that
 // share a kv head are multiplied against each K/V tile once, so KV is read from HBM once per step
 // instead of once per (worker, token) as in the reference (src/kernels/kernel_v21.cuh:62-66).
 //
@@ -10,7 +11,8 @@
 //   online softmax in base 2 on the accumulator layout (rows live on lane%16, so every per-row scalar
 //   is lane-local; only the row max needs two cross-lane steps)
 //   O^T[ev, row] += V^T[ev, token] . P^T[token, row]
-// K goes global -> VGPR straight into the A-operand layout (lane = token, 16 B of the head dim);
+// K goes global -> LDS by direct transfers (no VGPR staging) into a per-wave staging slot, XOR-swizzled so that
+// the A-operand reads (lane = token, 16 B of the head dim) are free of bank conflicts;
 // V is loaded as whole 256-byte rows (16 lanes x 16 B) and transposed in registers with v_perm_b32,
 // using the freedom to permute the reduced (token) index identically in both MFMA operands.
 // The query is rotated per fragment in the prologue (src/rope.cuh:18-51), rounded to the storage type
@@ -34,9 +36,6 @@ namespace hw {
 // waves per SIMD the two-row-block 16-bit kernels are register-budgeted for (tuning knob)
 #ifndef HW_MINW2
 #define HW_MINW2 1
-#endif
-#ifndef HW_VGPR_CAP
-#define HW_VGPR_CAP
 #endif
 
 // Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
@@ -64,7 +63,7 @@ namespace hw {
 // DEVLEN = the current fragment lengths come from device memory (header.len_dev); the lengths in the table are then
 // the bounds the split was planned for, and a captured launch stays valid while the segments grow up to them.
 template <class DT, int E, int EV, int RB, int MINW, int PF, bool PRE, bool DEVLEN = false, bool VS = false>
-__global__ __launch_bounds__(NTHREADS, MINW) HW_VGPR_CAP void attention_kernel(const KernelArgs args) {
+__global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     constexpr int ROWS = RB * 16;
 

@@ -25,6 +25,21 @@ def test_library_exports_every_declared_symbol():
     assert L.lib.hw_version() == 4
 
 
+def test_calibration_kernels_live_in_their_own_library():
+    """What only the benchmark needs is not part of the product ABI: libhogwild_bench.so exports what
+    include/hogwild_bench.h declares, and the product library exports none of it (no event or stream helpers either)."""
+    L = _lib()
+    header = open(os.path.join(ROOT, "include", "hogwild_bench.h")).read()
+    declared = set(re.findall(r"^\s*int\s+(hw_\w+)\s*\(", header, flags=re.M))
+    assert declared == {"hw_stream_read", "hw_stream_copy"}, declared
+    bench = C.CDLL(os.path.join(ROOT, "inference_lib_amd", "libhogwild_bench.so"))
+    for name in declared:
+        assert hasattr(bench, name), name
+        assert not hasattr(L.lib, name), f"{name} leaked into the product library"
+    for name in ("hw_event_create", "hw_event_record", "hw_event_elapsed_ms", "hw_stream_create"):
+        assert not hasattr(L.lib, name), name
+
+
 def test_struct_layout_matches_header():
     """ctypes mirror and C struct must agree; sizeof is probed through a tiny C program when gcc is around."""
     import shutil
