@@ -590,8 +590,9 @@ def bench_paged(args, dev, quick=False):
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM_GBS, 4),
-                     "traffic": load_traffic(("paged_attention_kernel/varlen" if varlen else "paged_attention_kernel/decode") + f"_{L}_{bs}"),
-                     "kernel": "hw::paged_attention_kernel",
+                     "traffic": load_traffic((("paged_wide_kernel" if plan.row_blocks == 8 else "paged_attention_kernel") +
+                                              ("/varlen" if varlen else "/decode")) + f"_{L}_{bs}"),
+                     "kernel": "hw::paged_wide_kernel" if plan.row_blocks == 8 else "hw::paged_attention_kernel",
                      "kernel_us_avg": round(kern_us, 3),
                      "kernel_us_p10_p90": [round(kern["p10"], 3), round(kern["p90"], 3)],
                      "timing": f"HIP event pairs around each of {kern['replays']} back-to-back replays of a graph of K attention-kernel launches "

@@ -188,7 +188,8 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
 
     hipError_t e = hipSuccess;
     if (stages & HW_STAGE_ATTENTION) {
-        e = hw::launch_paged_attention(ph, p->dtype, p->E, plan.row_blocks, stream);
+        if (plan.row_blocks == hw::WIDE_ROW_BLOCKS) e = hw::launch_paged_attention_wide(ph, p->dtype, p->E, stream);
+        else e = hw::launch_paged_attention(ph, p->dtype, p->E, plan.row_blocks, stream);
         if (e != hipSuccess) return (int)e;
     }
     if (!(stages & HW_STAGE_MERGE)) return (int)e;

@@ -8,6 +8,7 @@ constexpr int TILE = 32;       // tokens per wave step
 constexpr int NWAVES = 4;      // waves per workgroup
 constexpr int NTHREADS = NWAVES * 64;
 constexpr int WIDE_ROW_BLOCKS = 8;   // 16-row blocks of a workgroup of the many-rows kernel (32 rows per wave)
+constexpr int PAGED_WIDE_MAX_BLOCKS = 8192;   // block-table entries of one sequence the many-rows paged kernel keeps in LDS
 constexpr int MAX_SPLITS = 256;  // workgroups per kv head (size of the boundary table below)
 
 }  // namespace hw

@@ -581,6 +581,28 @@ struct DevHeader {
 };
 static_assert(sizeof(DevHeader) == sizeof(KernelHeader), "DevHeader mirrors KernelHeader");
 
+// PagedHeader as the paged kernels see it after fetching it by hand (see DevHeader).
+struct PagedDevHeader {
+    const HW_GLOBAL char* q;
+    const HW_GLOBAL int* loc;
+    const HW_GLOBAL int* frag_len;
+    const HW_GLOBAL char* kcache;
+    const HW_GLOBAL char* vcache;
+    const HW_GLOBAL int* block_table;
+    const HW_GLOBAL int* cu_q;
+    HW_GLOBAL float* part_o;
+    HW_GLOBAL float* part_ml;
+    int F, W, Hq, Hkv, LW, LS;
+    int R;
+    int block_size, max_blocks, num_blocks;
+    int nsplit, nitems, nrg, nwg;
+    int xcd_remap;
+    float sc;
+    unsigned magic_gq, magic_ls, magic_bs, magic_nsplit, magic_nitems, magic_nrg;
+};
+static_assert(sizeof(PagedDevHeader) == 160, "40 dwords of PagedHeader are fetched");
+static_assert(offsetof(PagedHeader, pad) == 160, "PagedDevHeader mirrors the used part of PagedHeader");
+
 // n / d for n < 2^20, d < 2^12 with the host-computed multiplier ceil(2^32 / d) mod 2^32: one multiply-high instead
 // of the ~25-instruction integer division sequence.  d == 1 gives the multiplier 0, which stands for "n itself".
 __device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }

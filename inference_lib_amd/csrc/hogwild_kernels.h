@@ -105,6 +105,7 @@ struct CopyBlocksArgs {
 };
 
 hipError_t launch_paged_attention(const PagedHeader& ph, int dtype, int E, int rb, hipStream_t stream);
+hipError_t launch_paged_attention_wide(const PagedHeader& ph, int dtype, int E, hipStream_t stream);   // 128 rows per workgroup
 hipError_t launch_copy_to_blocks(const CopyBlocksArgs& ca, int dtype, hipStream_t stream);
 
 // ---- caller-side steps: input builder and fused key rotation + append ----

@@ -33,27 +33,6 @@
 
 namespace hw {
 
-struct PagedDevHeader {
-    const HW_GLOBAL char* q;
-    const HW_GLOBAL int* loc;
-    const HW_GLOBAL int* frag_len;
-    const HW_GLOBAL char* kcache;
-    const HW_GLOBAL char* vcache;
-    const HW_GLOBAL int* block_table;
-    const HW_GLOBAL int* cu_q;
-    HW_GLOBAL float* part_o;
-    HW_GLOBAL float* part_ml;
-    int F, W, Hq, Hkv, LW, LS;
-    int R;
-    int block_size, max_blocks, num_blocks;
-    int nsplit, nitems, nrg, nwg;
-    int xcd_remap;
-    float sc;
-    unsigned magic_gq, magic_ls, magic_bs, magic_nsplit, magic_nitems, magic_nrg;
-};
-static_assert(sizeof(PagedDevHeader) == 160, "40 dwords of PagedHeader are fetched");
-static_assert(offsetof(PagedHeader, pad) == 160, "PagedDevHeader mirrors the used part of PagedHeader");
-
 template <class DT, int E, int EV, int RB, int MINW>
 __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const PagedHeader args) {
     typedef Geo<DT, E, EV> G;

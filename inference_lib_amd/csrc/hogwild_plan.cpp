@@ -207,8 +207,13 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     // more rows (several query tokens, wide GQA groups)
     const long long rows_per_worker = varlen ? (tokens * gq + p->W - 1) / p->W : (long long)p->S * gq;
     plan->row_blocks = rows_per_worker <= 16 ? 1 : 2;
-    if (p->row_blocks == 1 || p->row_blocks == 2) plan->row_blocks = p->row_blocks;
+    // many rows per sequence: 128-row workgroups whose waves share every K/V tile through LDS (16-bit types; the kernel
+    // keeps a sequence's block table in LDS, up to PAGED_WIDE_MAX_BLOCKS entries)
+    const bool wide_ok = p->dtype != HW_F32 && p->max_blocks <= hw::PAGED_WIDE_MAX_BLOCKS;
+    if (wide_ok && rows_per_worker > 64) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
+    if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
     if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
+    const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rpw = 16 * plan->row_blocks;
     long long items;
     if (varlen) items = p->W + tokens * gq / rpw;          // sum_w ceil(rows_w / rpw) <= W + rows / rpw
@@ -224,7 +229,11 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
         const long long pairs = (long long)p->Hkv * items;
         const long long tiles = ((long long)p->block_size * p->max_blocks + hw::TILE - 1) / hw::TILE;
         long long s, by_work;
-        if (2 * pairs <= num_cus) {
+        if (wide) {
+            // every wave takes every tile of its workgroup: fill the CUs once, at least four tiles per workgroup
+            s = pairs < num_cus ? num_cus / pairs : 1;
+            by_work = (tiles + 3) / 4;
+        } else if (2 * pairs <= num_cus) {
             s = num_cus / pairs;
             by_work = (tiles + hw::NWAVES - 1) / hw::NWAVES;
         } else {

@@ -414,6 +414,314 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     }
 }
 
+// One 1 KB global->LDS transfer with a 64-bit address per lane (the paged cache has no contiguous slice a buffer
+// descriptor could bound): lane l brings 16 bytes from `src` to LDS byte `lds` + 16 l, non-temporal.  Issued from inline
+// assembly and waited for by hand, like lds_transfer.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void lds_transfer_flat(unsigned lds, unsigned long long src) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds), "v"(src) : "m0", "memory");
+}
+#pragma clang diagnostic pop
+
+// The paged operators (hogwild_paged_sdpa / hogwild_varlen_paged_sdpa, see hogwild_paged.hip) for many query rows per
+// sequence: one workgroup = one kv head x one group of up to 128 rows of ONE sequence x every nsplit-th 32-token tile of
+// that sequence, with the tile ring of attention_wide_kernel.  What differs is where a tile's rows lie: position l of
+// sequence w is row l % block_size of block block_table[w][l / block_size] (src/kernels/kernel_v21.cuh:405-411).  The
+// sequence's block table is copied into LDS once (up to PAGED_WIDE_MAX_BLOCKS entries; the launcher sends longer tables
+// to the narrow kernel).  Per tile every lane derives the cache rows it fetches from it; positions no row of the group
+// can see are redirected to the last visible one (no byte outside the visible part of the sequence is read; block ids
+// are clamped into the cache).
+template <class DT, int E, int EV, int NS>
+__global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHeader args) {
+
+    typedef Geo<DT, E, EV> G;
+    constexpr int NW = NWAVES;
+    constexpr int NT = NTHREADS;
+    constexpr int RB = WIDE_ROWS / 16 / NW;
+    constexpr int WROWS = RB * 16;
+    constexpr int TPR = NT / WIDE_ROWS;
+    constexpr int D = NS - 2;
+    constexpr int KBYTES = G::KSTAGE;
+    constexpr int VBYTES = TILE * G::VROW;
+    constexpr int TPW = (KBYTES + VBYTES) / 1024 / NW;
+    constexpr int SLOT = KBYTES + VBYTES;
+    constexpr int RPL = 64 / G::CPR;             // tile rows one transfer covers
+    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && D >= 1 && NS >= 3 && G::KROW == G::VROW,
+                  "16-bit types; a wave's transfers belong to one image");
+
+    __shared__ __attribute__((aligned(16))) char q_lds[WIDE_ROWS * G::QSTR];
+    __shared__ int lim_lds[WIDE_ROWS];
+    __shared__ int bt_lds[PAGED_WIDE_MAX_BLOCKS];
+    __shared__ __attribute__((aligned(16))) char ring[NS * SLOT];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15;
+    const int q = lane >> 4;
+
+    typedef int i32x16 __attribute__((ext_vector_type(16)));
+    typedef int i32x8 __attribute__((ext_vector_type(8)));
+    struct HeaderBits {
+        i32x16 lo, mid;
+        i32x8 hi;
+    };
+    HeaderBits hb;
+    {
+        const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx8 %2, %3, 0x80"
+                     : "=&s"(hb.lo), "=&s"(hb.mid), "=&s"(hb.hi)
+                     : "s"(argp)
+                     : "memory");
+    }
+    // this wave's share of a tile's transfers: the first half of the waves fill the K image, the second half V
+    const bool k_wave = wv < NW / 2;
+    const int first = (k_wave ? wv : wv - NW / 2) * TPW;
+    const int lrow = lane / G::CPR, lslot = lane % G::CPR;
+    unsigned chunk[TPW];                          // byte offset of this lane's 16 bytes within its row, per transfer
+    int trow[TPW];                                // the tile row it belongs to
+#pragma unroll
+    for (int j = 0; j < TPW; ++j) {
+        const int row = (first + j) * RPL + lrow;
+        const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+        trow[j] = row;
+        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : lslot) << 4);
+    }
+    const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
+    WaveState<RB, G::NOC> st;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        st.m[rb] = NEG_BIG;
+        st.l[rb] = 0.f;
+#pragma unroll
+        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    st.fresh = true;
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.mid), "+s"(hb.hi) : : "memory");
+    struct RawHeader {
+        int v[40];
+    } raw;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        raw.v[i] = hb.lo[i];
+        raw.v[16 + i] = hb.mid[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw.v[32 + i] = hb.hi[i];
+    const PagedDevHeader ph = __builtin_bit_cast(PagedDevHeader, raw);
+
+    // logical workgroup id = ((kv head * nitems) + item) * nsplit + split; consecutive ids share an XCD
+    int bid = blockIdx.x;
+    if (ph.xcd_remap) bid = (bid & 7) * (ph.nwg >> 3) + (bid >> 3);
+    const int hi = fast_div(bid, ph.magic_nsplit);
+    const int split = bid - hi * ph.nsplit;
+    const int hkv = fast_div(hi, ph.magic_nitems);
+    const int item = hi - hkv * ph.nitems;
+    const int GQ = ph.Hq / ph.Hkv;
+
+    // item -> (worker, row group, query-token range of the worker), as in paged_attention_kernel
+    int w = 0, rg = 0, qs = 0, qe = 0;
+    if (ph.cu_q == nullptr) {
+        w = fast_div(item, ph.magic_nrg);
+        rg = item - w * ph.nrg;
+        qs = w * ph.LS;
+        qe = qs + ph.LS;
+    } else {
+        bool found = false;
+        int base = 0;
+        for (int c = 0; c < ph.W && !found; c += 64) {
+            const int idx = c + lane;
+            const int a0 = ph.cu_q[min(idx, ph.W)], a1 = ph.cu_q[min(idx + 1, ph.W)];
+            const int cnt = idx < ph.W ? (max(a1 - a0, 0) * GQ + WIDE_ROWS - 1) / WIDE_ROWS : 0;
+            int inc = cnt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int v = __shfl_up(inc, off, 64);
+                if (lane >= off) inc += v;
+            }
+            const int total = __builtin_amdgcn_readlane(inc, 63);
+            if (item < base + total) {
+                const int l0 = __builtin_ctzll(__ballot(base + inc > item));
+                w = c + l0;
+                rg = item - base - __builtin_amdgcn_readlane(inc - cnt, l0);
+                qs = __builtin_amdgcn_readlane(a0, l0);
+                qe = __builtin_amdgcn_readlane(a1, l0);
+                found = true;
+            }
+            base += total;
+        }
+        if (!found) return;   // the grid is sized for the worst case; uniform over the workgroup
+    }
+    const int T = ph.LW * ph.LS;
+    qe = min(qe, T);
+    qs = min(max(qs, 0), qe);
+    const int r0 = qs * GQ + rg * WIDE_ROWS;    // first row of the workgroup (global numbering: token * GQ + head in group)
+    const int rend = qe * GQ;                   // end of the worker's rows
+    if (r0 >= rend) return;                     // uniform over the workgroup
+    const int w0 = r0 + wv * WROWS;             // first row of this wave
+    const int cap = ph.block_size * ph.max_blocks;
+    const HW_GLOBAL int* btw = ph.block_table + (size_t)w * ph.max_blocks;
+    const unsigned long long image = reinterpret_cast<unsigned long long>(k_wave ? ph.kcache : ph.vcache);
+
+    DevHeader a;
+    a.q = ph.q;
+    a.loc = ph.loc;
+    a.cos = nullptr;
+    a.sin = nullptr;
+    a.rq = nullptr;
+    a.part_o = ph.part_o;
+    a.part_ml = ph.part_ml;
+    a.len_dev = nullptr;
+    a.F = ph.F; a.W = ph.LW; a.Hq = ph.Hq; a.Hkv = ph.Hkv; a.S = ph.LS; a.R = rend;
+    a.nrg = 1; a.wgs_per_head = ph.nsplit; a.nwg = ph.nwg;
+    a.prerotated = 1; a.xcd_remap = 0; a.sc = ph.sc;
+    a.magic_gq = ph.magic_gq; a.magic_s = ph.magic_ls; a.magic_nrg = 0; a.magic_wg = 0;
+
+    // The sequence's block table goes into LDS once: per tile every lane then looks up the block of its own position
+    // there.  (Read from memory per tile it is either a vector load, which the hand-counted tile transfers would have
+    // to wait behind, or a scalar load, whose latency every LDS wait of the tile loop then inherits: measured, 0.4 us
+    // per tile.)
+    {
+        const int nent = min(ph.max_blocks, PAGED_WIDE_MAX_BLOCKS);
+        for (int i = tid; i < nent; i += NT) bt_lds[i] = btw[i];
+    }
+
+    for (int f = 0; f < ph.F; ++f) {
+        QueryRotation<DT, E, WIDE_ROWS, G::QSTR, true, NT> qrot;
+        qrot.load(a, f, hkv, r0, GQ, tid);
+        const int lm = ph.loc[(size_t)f * T + fast_div(min(r0 + tid / TPR, rend - 1), ph.magic_gq)];
+        const int flen = ph.frag_len[ph.cu_q != nullptr ? f * ph.W + w : f];
+
+        __syncthreads();   // the previous fragment's readers are done with q_lds / lim_lds / the ring
+        qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tid);
+        if (tid % TPR == 0) lim_lds[tid / TPR] = (r0 + tid / TPR < rend) ? max(0, min(min(flen, cap), lm < cap ? lm + 1 : cap)) : 0x7fffffff;
+        __syncthreads();
+
+        u32x4 qreg[RB * G::KJ];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+            for (int j = 0; j < G::KJ; ++j)
+                qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * WROWS + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+        int lim[RB];
+        int maxlim = 0, minlim = 0x7fffffff;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            lim[rb] = lim_lds[wv * WROWS + rb * 16 + n];
+            const bool pad = w0 + rb * 16 + n >= rend;
+            maxlim = max(maxlim, pad ? 0 : lim[rb]);
+            minlim = min(minlim, lim[rb]);
+        }
+#pragma unroll
+        for (int off = 1; off < 16; off <<= 1) {
+            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
+            minlim = min(minlim, __shfl_xor(minlim, off, 64));
+        }
+        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
+        minlim = __builtin_amdgcn_readfirstlane(minlim);
+        // what the WORKGROUP can see decides which positions are fetched and where its tile loop ends (every wave must
+        // take part in every tile's barrier); what the wave can see decides which tiles it multiplies
+        int wgmax = 0;
+#pragma unroll
+        for (int i = 0; i < WIDE_ROWS / 64; ++i) {
+            const int r = i * 64 + lane;
+            wgmax = max(wgmax, r0 + r < rend ? lim_lds[r] : 0);
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) wgmax = max(wgmax, __shfl_xor(wgmax, off, 64));
+        wgmax = __builtin_amdgcn_readfirstlane(wgmax);
+
+        // Source addresses of this wave's share of tile t (TPW transfers): every lane looks up the block of the row it
+        // fetches in each transfer.  A position beyond what the workgroup can see is replaced by the last visible one, so a
+        // tile that does not exist costs the same number of transfers and no new memory traffic to speak of, and no byte
+        // outside the visible part of the sequence is read.
+        auto addresses = [&](unsigned long long* src, int t) {
+#pragma unroll
+            for (int j = 0; j < TPW; ++j) {
+                const int tok = min(t * TILE + trow[j], wgmax - 1);
+                const int bi = fast_div(tok, ph.magic_bs);
+                const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
+                const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
+                src[j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
+            }
+        };
+        auto request = [&](int sl, const unsigned long long* src) {
+#pragma unroll
+            for (int j = 0; j < TPW; ++j) lds_transfer_flat(my_image + sl * SLOT + j * 1024, src[j]);
+        };
+
+        if (wgmax > 0) {   // uniform over the workgroup
+            // tiles of this workgroup: split, split + nsplit, ...  The addresses of a request are formed one tile earlier
+            // (after the barrier, next to the arithmetic): the request at the top of a tile is then four transfers and
+            // nothing else, and no wave reaches the barrier late because it was still looking up blocks.
+            const int ns = ph.nsplit;
+            unsigned long long src[TPW];
+#pragma unroll
+            for (int i = 0; i < D; ++i) {
+                addresses(src, split + i * ns);
+                request(i, src);
+            }
+            addresses(src, split + D * ns);
+            bool done = false;
+            for (int k0 = 0; !done; k0 += NS) {
+#pragma unroll
+                for (int i = 0; i < NS; ++i) {
+                    const int t = split + (k0 + i) * ns;
+                    if (t * TILE >= wgmax) {      // uniform over the workgroup: every wave leaves at the same tile
+                        done = true;
+                        break;
+                    }
+                    request((i + D) % NS, src);   // tile t + D * ns
+                    // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
+                    // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
+                    addresses(src, t + (D + 1) * ns);
+                    const int t0 = t * TILE;
+                    if (t0 < maxlim) {
+                        const char* slot = ring + i * SLOT;
+                        TileRegs<DT, E, EV> tr;
+                        read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
+                        if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, ph.sc, slot);
+                        else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, ph.sc, slot);
+                    }
+                }
+            }
+            // the requests behind the last tile must have landed before the ring is used again
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    }
+
+    // ---- every wave stores the partial of its own rows, 16-row blocks staged through the ring (see attention_wide_kernel) ----
+    {
+        constexpr int OSTR = EV + 4;
+        static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+        __syncthreads();
+        float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const float lsum = quarter_sum(st.l[rb]);
+            const int row0 = w0 + rb * 16;
+            const size_t prow0 = (size_t)(hkv * ph.nsplit + split) * ph.R + row0;
+#pragma unroll
+            for (int c0 = 0; c0 < G::NOC; c0 += 4)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    *reinterpret_cast<f32x4*>(stage + n * OSTR + out_ev<DT, EV>(c0, 4 * q + i)) =
+                        f32x4{st.o[rb][c0][i], st.o[rb][c0 + 1][i], st.o[rb][c0 + 2][i], st.o[rb][c0 + 3][i]};
+            if (q == 0 && row0 + n < rend) *reinterpret_cast<HW_GLOBAL f32x2*>(ph.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
+            const int nvalid = min(16, rend - row0);
+            HW_GLOBAL float* dst = ph.part_o + prow0 * EV;
+#pragma unroll
+            for (int ps = 0; ps < 16 * EV / 256; ++ps) {
+                const int idx = ps * 256 + lane * 4;
+                const int rr = idx / EV, e = idx % EV;
+                if (rr < nvalid) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * OSTR + e);
+            }
+        }
+    }
+}
+
 // Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
 // usual cure for a loop that waits) double what the waves read out of LDS per tile, and the kernel got slower by a
 // tenth (27.3 against 24.7 us at 128 rows x 16 K tokens x 8 kv heads, fp16).
@@ -444,4 +752,22 @@ hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStre
     }
 }
 
+template <class DT>
+static hipError_t launch_paged_wide_dt(const PagedHeader& ph, int E, hipStream_t stream) {
+    constexpr int NS = 5;      // ring slots: 5, 6 and 7 measure the same (a wave waits 4 ns per tile for its own transfers)
+    if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS>), dim3(ph.nwg), dim3(NTHREADS), 0, stream, ph);
+    else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS>), dim3(ph.nwg), dim3(NTHREADS), 0, stream, ph);
+    return hipGetLastError();
+}
+
+hipError_t launch_paged_attention_wide(const PagedHeader& ph, int dtype, int E, hipStream_t stream) {
+    if (ph.max_blocks > PAGED_WIDE_MAX_BLOCKS) return hipErrorInvalidValue;   // the table of a sequence must fit into LDS
+    switch (dtype) {
+        case 1: return launch_paged_wide_dt<F16>(ph, E, stream);
+        case 2: return launch_paged_wide_dt<BF16>(ph, E, stream);
+        default: return hipErrorInvalidValue;     // 16-bit types only
+    }
+}
+
 }  // namespace hw
+

@@ -256,21 +256,33 @@ def test_paged_plan_invariants():
     # short sequences: never more waves than tiles at the longest sequence the table allows
     pl = L.paged_plan(W=1, Hq=8, Hkv=8, Ev=128, block_size=16, max_blocks=8, num_cus=256, S=1)
     assert pl.splits == 1
-    # many query tokens per worker: two row blocks, several row groups
+    # several query tokens per worker: two row blocks, several row groups
+    pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=12)
+    assert pl.row_blocks == 2 and pl.row_groups == 2 * 2
+    # more than 64 rows per worker: 128-row workgroups (16-bit types, at most 8192 table entries per sequence), the CUs filled once
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20)
+    assert pl.row_blocks == 8 and pl.row_groups == 2 * 1 and pl.splits == 8 and pl.workgroups == 128   # 32 tiles: four per workgroup at least
+    pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=1, max_blocks=9000, num_cus=256, S=20)   # table too long for LDS
+    assert pl.row_blocks == 2 and pl.row_groups == 2 * 4
+    pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20, row_blocks=2)
     assert pl.row_blocks == 2 and pl.row_groups == 2 * 4
     # fp32 exists with one row block only
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20, dtype=L.HW_F32)
     assert pl.row_blocks == 1 and pl.row_groups == 2 * 7
     # variable length: the row-group count is an upper bound over every way of cutting total_q into W sequences
-    pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700)
+    pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700, row_blocks=2)
     assert pl.rows == 3500 and pl.row_groups >= 8 + 3500 // 32 and pl.workgroups == 8 * pl.row_groups * pl.splits
+    pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700)
+    assert pl.row_blocks == 8 and pl.row_groups >= 8 + 3500 // 128 and pl.workgroups == 8 * pl.row_groups * pl.splits
     # more (kv head, row group) pairs than half the CUs: about three workgroups per CU on long sequences, no
     # splitting at all on short ones or when the pairs alone oversubscribe the chip that far
-    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105, row_blocks=2)
     assert pl.row_groups == 20 and pl.splits == 5 and 3 * 256 <= pl.workgroups < 4 * 256
-    assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=30, num_cus=256, total_q=105).splits == 1
+    assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=30, num_cus=256, total_q=105, row_blocks=2).splits == 1
     assert L.paged_plan(W=64, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=640).splits == 1
+    # the same packed queries in 128-row workgroups: 8 row groups at most, the CUs filled once
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
+    assert pl.row_blocks == 8 and pl.row_groups == 8 and pl.splits == 4 and pl.workgroups == 256
     # explicit split factor is honoured (capped at 64)
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=5).splits == 5
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=500).splits == 64

@@ -140,6 +140,44 @@ def test_paged_gqa16_and_wide_rows():
     check(c)
 
 
+@pytest.mark.parametrize("dtype,D,bs,S,F,splits", [
+    ("bf16", 128, 16, 7, 1, 0),      # 112 rows per sequence: chosen automatically
+    ("f16", 128, 24, 9, 2, 3),       # blocks of 24 positions: a tile touches three blocks; two fragments
+    ("bf16", 64, 128, 3, 1, 1),      # forced with few rows (48), one split
+    ("f16", 64, 17, 20, 1, 7),       # 320 rows: three row groups, the last partly filled; odd block size
+])
+def test_paged_wide_rows(dtype, D, bs, S, F, splits):
+    """The 128-row workgroups of the paged operators (row_blocks = 8) against the oracle."""
+    c = build_paged(dtype, F, 3, 32, 2, D, bs, (700 + bs - 1) // bs + 1, seq_lens=[700, 131, 64], S=S, seed=31 + bs)
+    check(c, splits=splits, row_blocks=8)
+    c = build_paged(dtype, F, 2, 32, 2, D, bs, (300 + bs - 1) // bs + 1, seq_lens=[300, 290], S=S, seed=5, loc_mode="random")
+    check(c, splits=splits, row_blocks=8)
+
+
+def test_varlen_wide_rows():
+    """Packed variable-length queries with many tokens per sequence: 5 .. 1000 rows per kv head and sequence, empty and
+    one-token sequences in between, sequences shorter than a tile."""
+    c = build_paged("bf16", 1, 6, 10, 2, 128, 16, 60, seq_lens=[900, 50, 9, 430, 64, 777], q_lens=[200, 0, 9, 64, 1, 33], seed=77)
+    check(c)                              # 511 rows / 6 sequences: the planner picks the wide kernel by itself
+    check(c, row_blocks=8, splits=5)
+    check(c, row_blocks=2)                # and the narrow kernel agrees with the same oracle
+    c = build_paged("f16", 2, 3, 8, 2, 64, 32, 20, seq_lens=[600, 31, 222], q_lens=[100, 31, 64], seed=3, loc_mode="random")
+    check(c, row_blocks=8)
+
+
+def test_paged_wide_small_blocks_and_fallbacks():
+    """Any block size works in the 128-row workgroups (the table is looked up per position); fp32 and block tables that do
+    not fit into LDS (more than 8192 entries per sequence) have no such kernel: the request is ignored, never a wrong launch."""
+    c = build_paged("bf16", 1, 2, 32, 2, 128, 8, 40, seq_lens=[300, 200], S=6, seed=2)
+    check(c, row_blocks=8)
+    c = build_paged("f16", 2, 2, 16, 2, 64, 1, 150, seq_lens=[150, 77], S=9, seed=4)
+    check(c, row_blocks=8)
+    c = build_paged("f32", 1, 2, 32, 2, 64, 16, 20, seq_lens=[300, 200], S=6, seed=2)
+    check(c, row_blocks=8)
+    c = build_paged("bf16", 1, 1, 32, 2, 64, 1, 8200, seq_lens=[8195], S=6, seed=6, poison=False)
+    check(c, row_blocks=8)
+
+
 def test_paged_nothing_visible():
     c = build_paged("bf16", 1, 2, 4, 2, 64, 16, 4, seq_lens=[20, 20], S=1, seed=1)
     c["loc"][:, 0] = -1
