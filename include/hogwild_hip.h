@@ -219,7 +219,7 @@ typedef struct hw_paged_problem {
     void* workspace;
     size_t workspace_bytes;
     int32_t splits;            /* 0 = automatic; otherwise workgroups per (kv head, row group) */
-    int32_t row_blocks;        /* 0 = automatic; 1 or 2 = 16-row MFMA blocks per workgroup */
+    int32_t row_blocks;        /* 0 = automatic; 1, 2 or 8 = 16-row MFMA blocks per workgroup (8: 128-row workgroups, 16-bit types, max_blocks <= 8192) */
 } hw_paged_problem;
 
 typedef struct hw_paged_plan {
