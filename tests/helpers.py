@@ -39,7 +39,7 @@ def oracle_fused(oracle, case, second_half_index="first"):
     return out, lse, rq
 
 
-def run_fused(case_dev, *, splits=0, with_rq=True, with_lse=True):
+def run_fused(case_dev, *, splits=0, with_rq=True, with_lse=True, row_blocks=0):
     """Call hw_fused_attention through the C ABI on a Case whose tensors are on the GPU."""
     from inference_lib_amd import _lib
     dev = case_dev.q.device
@@ -48,7 +48,8 @@ def run_fused(case_dev, *, splits=0, with_rq=True, with_lse=True):
     lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=dev) if with_lse else None
     rq = torch.full((case_dev.F, W, Hq, S, E), float("nan"), dtype=case_dev.q.dtype, device=dev) if with_rq else None
     pr = _lib.Problem(q=case_dev.q, locations=case_dev.locations, keys=case_dev.keys, values=case_dev.values,
-                      scale=case_dev.scale, out=out, cosines=case_dev.cos, sines=case_dev.sin, rq=rq, lse=lse, splits=splits)
+                      scale=case_dev.scale, out=out, cosines=case_dev.cos, sines=case_dev.sin, rq=rq, lse=lse, splits=splits,
+                      row_blocks=row_blocks)
     pr.run()
     torch.cuda.synchronize()
     return out, lse, rq

@@ -71,6 +71,58 @@ def test_paged_random_shapes(seed):
     check_paged(c, splits=int(rng.choice([0, 0, 1, 5])))
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_wide_random_shapes(oracle, seed):
+    """The 128-row workgroups (row_blocks = 8) on random shapes: 16-bit types, 1..9 workers x 1..6 tokens x GQA 1..8, i.e.
+    from a single row to several row groups, fragments around the tile size, empty fragments, explicit split factors."""
+    from inference_lib_amd import cases
+    rng = np.random.default_rng(7000 + seed)
+    dtype = ["bf16", "f16"][seed % 2]
+    E = [128, 64][(seed // 2) % 2]
+    W, S = int(rng.integers(1, 10)), int(rng.integers(1, 7))
+    Hkv, GQ = int(rng.choice([1, 2, 4])), int(rng.integers(1, 9))
+    F = int(rng.integers(1, 9))
+    lens = [int(rng.choice(EDGE)) if rng.random() < 0.7 else int(rng.integers(0, 2000)) for _ in range(F)]
+    if sum(lens) == 0:
+        lens[0] = 33
+    orders = [[int(x) for x in rng.permutation(F)] for _ in range(W)]
+    c = cases.build_case(f"wide{seed}", dtype, W, S, Hkv * GQ, Hkv, E, 1e4, lens, orders, torch.Generator().manual_seed(seed))
+    splits = int(rng.choice([0, 0, 1, 3, 9]))
+    print(f"seed {seed}: {dtype} E={E} W={W} S={S} Hq={Hkv * GQ} Hkv={Hkv} rows={W * S * GQ} lens={lens} splits={splits}", flush=True)
+    want_o, want_l, want_rq = oracle_fused(oracle, c)
+    out, lse, rq = run_fused(c.to(torch.device("cuda:0")), splits=splits, row_blocks=8)
+    assert_close("out", out, want_o, TOL[dtype])
+    assert_close("lse", lse, want_l, TOL[dtype])
+    assert_close("rq", rq, want_rq, 3.2e-2)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_paged_wide_random_shapes(seed):
+    """The 128-row workgroups of the paged operators on random shapes: up to 24 query tokens per sequence (fixed) or 0..60
+    (packed), any block size, several fragments, random and causal locations."""
+    rng = np.random.default_rng(9000 + seed)
+    dtype = ["bf16", "f16"][seed % 2]
+    D = [128, 64][(seed // 2) % 2]
+    W = int(rng.integers(1, 6))
+    Hkv, GQ = int(rng.choice([1, 2, 4])), int(rng.integers(1, 9))
+    bs = int(rng.choice([1, 5, 16, 16, 32, 100, 256]))
+    F = int(rng.integers(1, 4))
+    varlen = bool(rng.random() < 0.5)
+    S = int(rng.integers(1, 25))
+    longest = int(rng.choice([90, 400, 1500]))
+    seq = [int(rng.integers(64 + 3 * F, longest + 64 + 3 * F)) for _ in range(W)]
+    mb = (max(seq) + bs - 1) // bs + int(rng.integers(0, 3))
+    kw = dict(seed=seed, loc_mode="random" if rng.random() < 0.5 else "causal")
+    if varlen:
+        ql = [int(min(s - 3 * F, x)) for s, x in zip(seq, rng.integers(0, 61, size=W))]
+        if sum(ql) == 0:
+            ql[0] = 1
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, D, bs, mb, seq_lens=seq, q_lens=ql, **kw)
+    else:
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, D, bs, mb, seq_lens=[max(s, S + 3 * F + 1) for s in seq], S=S, **kw)
+    check_paged(c, splits=int(rng.choice([0, 0, 1, 5])), row_blocks=8)
+
+
 @pytest.mark.parametrize("seed", range(18))
 def test_fused_random_shapes_with_device_lengths(oracle, seed):
     """The same sweep through the device-resident-lengths path: every fragment sits in a buffer that is longer than
