@@ -1,7 +1,7 @@
 // Hogwild! fragmented-KV decode attention for gfx950 (MI355X, CDNA4, wave64).
 //
 // One workgroup = one kv head x one contiguous range of 32-token tiles (crossing fragment boundaries)
-// x up to 32 query rows, where a "row" is one (worker, token, q-head-in-group) triple (more than 64 rows per
+// x up to 32 query rows, where a "row" is one (worker, token, q-head-in-group) triple (more than 96 rows per
 // kv head: attention_wide_kernel, hogwild_wide.hip).  All rows that
 // share a kv head are multiplied against each K/V tile once, so KV is read from HBM once per step
 // instead of once per (worker, token) as in the reference (src/kernels/kernel_v21.cuh:62-66).

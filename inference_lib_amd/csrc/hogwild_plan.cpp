@@ -70,13 +70,13 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     if ((long long)p->Hkv * ((rows_ll + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
     const int rows = (int)rows_ll;
     plan->rows = rows;
-    // up to 16 rows: one 16-row block per workgroup (two workgroups per CU); up to 64: two blocks, rows beyond 32 in a
-    // second row group that reads the same KV; more: 128-row workgroups whose four waves share every K/V tile through
+    // up to 16 rows: one 16-row block per workgroup (two workgroups per CU); up to 96: two blocks, rows beyond 32 in
+    // further row groups that read the same KV; more: 128-row workgroups whose four waves share every K/V tile through
     // LDS (16-bit types, lengths known on the host) -- a CU can take in about 16 B/clk, so what counts is that every
     // CU reads every byte once
     const bool wide_ok = p->dtype != HW_F32 && p->len_dev == nullptr && p->variant == HW_VARIANT_MFMA;
     plan->row_blocks = rows <= 16 ? 1 : 2;
-    if (wide_ok && rows > 64) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
+    if (wide_ok && rows > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;   // measured crossover: 80 rows 24.6 (narrow) / 25.6 us, 120 rows 28.0 / 27.4 us
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rows_per_wg = 16 * plan->row_blocks;
@@ -210,7 +210,7 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     // many rows per sequence: 128-row workgroups whose waves share every K/V tile through LDS (16-bit types; the kernel
     // keeps a sequence's block table in LDS, up to PAGED_WIDE_MAX_BLOCKS entries)
     const bool wide_ok = p->dtype != HW_F32 && p->max_blocks <= hw::PAGED_WIDE_MAX_BLOCKS;
-    if (wide_ok && rows_per_worker > 64) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
+    if (wide_ok && rows_per_worker > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
     if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;

@@ -259,7 +259,7 @@ def test_paged_plan_invariants():
     # several query tokens per worker: two row blocks, several row groups
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=12)
     assert pl.row_blocks == 2 and pl.row_groups == 2 * 2
-    # more than 64 rows per worker: 128-row workgroups (16-bit types, at most 8192 table entries per sequence), the CUs filled once
+    # more than 96 rows per worker: 128-row workgroups (16-bit types, at most 8192 table entries per sequence), the CUs filled once
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20)
     assert pl.row_blocks == 8 and pl.row_groups == 2 * 1 and pl.splits == 8 and pl.workgroups == 128   # 32 tiles: four per workgroup at least
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=1, max_blocks=9000, num_cus=256, S=20)   # table too long for LDS

@@ -158,7 +158,7 @@ def test_varlen_wide_rows():
     """Packed variable-length queries with many tokens per sequence: 5 .. 1000 rows per kv head and sequence, empty and
     one-token sequences in between, sequences shorter than a tile."""
     c = build_paged("bf16", 1, 6, 10, 2, 128, 16, 60, seq_lens=[900, 50, 9, 430, 64, 777], q_lens=[200, 0, 9, 64, 1, 33], seed=77)
-    check(c)                              # 511 rows / 6 sequences: the planner picks the wide kernel by itself
+    check(c)                              # 511 rows / 6 sequences = 85 on average: the planner stays with the 32-row kernel
     check(c, row_blocks=8, splits=5)
     check(c, row_blocks=2)                # and the narrow kernel agrees with the same oracle
     c = build_paged("f16", 2, 3, 8, 2, 64, 32, 20, seq_lens=[600, 31, 222], q_lens=[100, 31, 64], seed=3, loc_mode="random")

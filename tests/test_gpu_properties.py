@@ -246,7 +246,7 @@ def test_graph_replay_matches_eager():
     ("bf16", 128, 2, 40, 8, 2, (500, 100, 120)),              # 40 query tokens per worker (prefill-like), 320 rows
 ])
 def test_wide_kernel_against_oracle(oracle, dtype, E, W, S, Hq, Hkv, lens):
-    """The 128-row workgroups (row_blocks = 8; chosen automatically beyond 64 rows per kv head) against the oracle, and
+    """The 128-row workgroups (row_blocks = 8; chosen automatically beyond 96 rows per kv head) against the oracle, and
     bit-identical to nothing: the narrow kernel sums in another order, so both are compared with the oracle."""
     from inference_lib_amd import _lib, cases
     c = cases.small_case(dtype=dtype, W=W, S=S, Hq=Hq, Hkv=Hkv, E=E, lens=lens, seed=len(lens) + W)
