@@ -488,13 +488,17 @@ def main():
         for cid in (1, 2, 4, 5):
             if cid != args.case:
                 cfgs.append(side_config(cid, dev, args, stream))
-        pargs = argparse.Namespace(**vars(args))
-        pargs.workload, pargs.no_cpu = "paged", True
-        pg = bench_paged(pargs, dev, quick=True)
-        cfgs.append({"workload": pg["config"]["workload"], "kv_bytes_per_step": pg["config"]["kv_bytes_per_step"],
-                     "workgroups": pg["config"]["workgroups"], "kernel_us": pg["roofline"]["kernel_us_avg"],
-                     "step_us": pg["extra"]["us_per_step"], "step_us_p10_p90": pg["extra"]["us_per_step_p10_p90"],
-                     "kernel_frac_of_peak": pg["roofline"]["frac"], "step_GBps": pg["value"]})
+        for wl in ("paged", "varlen"):
+            pargs = argparse.Namespace(**vars(args))
+            pargs.workload, pargs.no_cpu = wl, True
+            pg = bench_paged(pargs, dev, quick=True)
+            cfgs.append({"workload": pg["config"]["workload"], "kv_bytes_per_step": pg["config"]["kv_bytes_per_step"],
+                         "workgroups": pg["config"]["workgroups"], "kernel": pg["roofline"]["kernel"],
+                         "kernel_us": pg["roofline"]["kernel_us_avg"],
+                         "step_us": pg["extra"]["us_per_step"], "step_us_p10_p90": pg["extra"]["us_per_step_p10_p90"],
+                         "kernel_frac_of_peak": pg["roofline"]["frac"], "step_GBps": pg["value"]})
+            del pg
+            torch.cuda.empty_cache()
         result["extra"]["configs"] = cfgs
 
     if baseline is not None:
