@@ -156,7 +156,8 @@ int hw_fused_attention(const hw_problem* p, void* stream);
  * hw_fused_attention, except that p->workspace / p->workspace_bytes are ignored: the split-K partials go to a
  * device array that is part of the library image (HW_STATIC_SCRATCH_BYTES per GPU, resident until the process ends).
  * The call allocates and frees nothing.  A problem whose hw_workspace_bytes() exceeds HW_STATIC_SCRATCH_BYTES is
- * refused with HW_ERR_STATIC_SCRATCH before anything is queued.  All calls on one GPU share that GPU's array: calls
+ * refused with HW_ERR_STATIC_SCRATCH before anything is queued -- except that with row_blocks = 0 a plan of 128-row
+ * workgroups that does not fit is replaced by the 32-row kernel's (fewer partials), and only that one has to fit.  All calls on one GPU share that GPU's array: calls
  * that overlap in time on one GPU (different streams, or graphs replayed concurrently) race on the partials and
  * must be serialised by the caller.  Nothing in the array has to survive between calls or start at zero.
  */

@@ -406,13 +406,20 @@ int hw_fused_attention_static(const hw_problem* p, void* stream) {
     st = device_cus(&cus);
     if (st != HW_OK) return st;
     hw_plan plan;
-    st = make_plan(p, cus, &plan);
+    hw_problem q = *p;
+    st = make_plan(&q, cus, &plan);
     if (st != HW_OK) return st;
+    if (plan.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES && p->row_blocks == 0 && plan.row_blocks == hw::WIDE_ROW_BLOCKS) {
+        // the 128-row workgroups write a partial per split for all rows of a kv head: the 32-row kernel needs a quarter
+        // of that with its fewer splits per row group, and the caller left the choice to the library
+        q.row_blocks = 2;
+        st = make_plan(&q, cus, &plan);
+        if (st != HW_OK) return st;
+    }
     if (plan.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES) return HW_ERR_STATIC_SCRATCH;
     void* ptr = nullptr;
     st = static_scratch(&ptr);
     if (st != HW_OK) return st;
-    hw_problem q = *p;
     q.workspace = ptr;
     q.workspace_bytes = (size_t)HW_STATIC_SCRATCH_BYTES;
     return run(&q, stream, 1);

@@ -71,6 +71,39 @@ def test_static_scratch_partial_rotary_uses_the_array_for_the_rotated_queries(or
     assert_close("out", outs[1], o_ref, TOL[c.dtype])
 
 
+def test_static_scratch_takes_the_kernel_with_fewer_partials(oracle):
+    """128 rows per kv head: the 128-row workgroups would need 17 MB of partials, more than the array holds.  Left the
+    choice (row_blocks = 0), the entry point plans the 32-row kernel instead (4.3 MB) and gives bit for bit what the
+    workspace entry point gives with row_blocks = 2."""
+    from inference_lib_amd import _lib, cases
+    c = cases.baseline_case(5)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    res = []
+    for static in (False, True):
+        out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+        lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+        pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out,
+                          cosines=cd.cos, sines=cd.sin, lse=lse, row_blocks=0 if static else 2)
+        if static:
+            assert pr.workspace_bytes() > _lib.HW_STATIC_SCRATCH_BYTES      # what the automatic plan would need
+            pr.run_static()
+        else:
+            pr.run()
+        torch.cuda.synchronize()
+        res.append((out, lse))
+    assert torch.equal(res[0][0], res[1][0]) and torch.equal(res[0][1], res[1][1])
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", res[1][0], o_ref, TOL[c.dtype])
+    assert_close("lse", res[1][1], l_ref, TOL[c.dtype])
+    # asked for by name, the 128-row workgroups are refused: the caller's choice is not overridden
+    pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=res[1][0],
+                      cosines=cd.cos, sines=cd.sin, row_blocks=8)
+    with pytest.raises(_lib.HogwildError) as ei:
+        pr.run_static()
+    assert ei.value.status == -9
+
+
 def test_static_scratch_refuses_what_does_not_fit():
     """A problem whose partials exceed the array is refused on the host, before anything is queued."""
     from inference_lib_amd import _lib
