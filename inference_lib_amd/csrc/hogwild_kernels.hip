@@ -24,6 +24,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../../include/hogwild_hip.h"
 #include "hogwild_kernels.h"
 
@@ -281,29 +283,37 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 // Latency-bound, so everything a thread needs from global memory (its partial rows and their max/sum pairs) is
 // requested in one batch before the first use; each thread then folds its partials with a running reference of
 // its own, and the NPG partial groups are combined through LDS.
-template <class DT, int EV>
+// RPW = rows per workgroup: with few partials per row (at most 4 * NPG / RPW) a workgroup merges RPW rows side by side,
+// each with its share of the partial groups, instead of leaving most of its threads without a partial to load.
+template <class DT, int EV, int RPW>
 __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     typedef typename Elem<DT>::store_t store_t;
     constexpr int V4 = EV / 4;          // threads along the head dim (4 floats each)
-    constexpr int NPG = 256 / V4;       // partial groups
+    constexpr int NPG = 256 / V4;       // partial groups of the workgroup
+    constexpr int GPR = NPG / RPW;      // partial groups per row
     constexpr int UN = 4;               // partials per thread and batch
+    static_assert(GPR >= 1 && GPR * RPW == NPG, "the partial groups are dealt evenly to the rows");
     __shared__ __attribute__((aligned(16))) float red[NPG][EV];
     __shared__ float red_m[NPG], red_l[NPG];
 
     // Workgroups are dealt round-robin over the 8 XCDs.  When the attention kernel kept each kv head on one XCD, merge
     // that head's rows on the same XCD: its partials are then still in that XCD's L2.
-    int hkv, r;
+    const int nrb = (a.R + RPW - 1) / RPW;                // row blocks per kv head
+    int hkv, rblk;
     if (a.xcd_local) {
         const int hpx = a.Hkv >> 3;                       // heads per XCD
         const int x = blockIdx.x & 7, j = blockIdx.x >> 3;
         hkv = x * hpx + j % hpx;
-        r = j / hpx;
+        rblk = j / hpx;
     } else {
-        hkv = blockIdx.x / a.R;
-        r = blockIdx.x - hkv * a.R;
+        hkv = blockIdx.x / nrb;
+        rblk = blockIdx.x - hkv * nrb;
     }
     const int tid = threadIdx.x;
     const int e4 = tid % V4, pg = tid / V4;
+    const int rr = pg / GPR, pgl = pg % GPR;               // row within the workgroup, partial group within the row
+    const bool live = rblk * RPW + rr < a.R;
+    const int r = live ? rblk * RPW + rr : a.R - 1;        // (a row that does not exist re-reads the last one and stores nothing)
     const int ns = a.wgs_per_head;
     const float* ml = a.part_ml + ((size_t)hkv * ns * a.R + r) * 2;
     const size_t mstride = (size_t)a.R * 2;
@@ -312,13 +322,13 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
 
     float m_run = NEG_BIG, l_run = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = pg; s0 < ns; s0 += UN * NPG) {
+    for (int s0 = pgl; s0 < ns; s0 += UN * GPR) {
         f32x4 o[UN];
         f32x2 mlv[UN];
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const int s = s0 + u * NPG;
-            const int sc = s < ns ? s : pg;                 // clamp: the loads stay unconditional
+            const int s = s0 + u * GPR;
+            const int sc = s < ns ? s : pgl;                // clamp: the loads stay unconditional
             o[u] = *reinterpret_cast<const f32x4*>(po + (size_t)sc * ostride);
             mlv[u] = *reinterpret_cast<const f32x2*>(ml + (size_t)sc * mstride);
             if (s >= ns) mlv[u] = f32x2{NEG_BIG, 0.f};
@@ -343,17 +353,18 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
         red_l[pg] = l_run;
     }
     __syncthreads();
-    if (pg == 0) {
-        float M = red_m[0];
+    if (pgl == 0 && live) {
+        const int g0 = rr * GPR;                           // this row's partial groups: g0 .. g0 + GPR - 1
+        float M = red_m[g0];
 #pragma unroll
-        for (int k = 1; k < NPG; ++k) M = fmaxf(M, red_m[k]);
+        for (int k = 1; k < GPR; ++k) M = fmaxf(M, red_m[g0 + k]);
         f32x4 tot = {0.f, 0.f, 0.f, 0.f};
         float L = 0.f;
 #pragma unroll
-        for (int k = 0; k < NPG; ++k) {
-            const float w = fast_exp2(red_m[k] - M);
-            tot += *reinterpret_cast<const f32x4*>(&red[k][e4 * 4]) * w;
-            L += red_l[k] * w;
+        for (int k = 0; k < GPR; ++k) {
+            const float w = fast_exp2(red_m[g0 + k] - M);
+            tot += *reinterpret_cast<const f32x4*>(&red[g0 + k][e4 * 4]) * w;
+            L += red_l[g0 + k] * w;
         }
         const float inv = L > 0.f ? 1.0f / L : 0.f;
         const int GQ = a.Hq / a.Hkv;
@@ -446,14 +457,27 @@ hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, int 
     }
 }
 
+template <class DT, int EV>
+static hipError_t launch_merge_ev(const MergeArgs& ma, hipStream_t stream) {
+    constexpr int NPG = 256 / (EV / 4);
+    // rows per workgroup: as many as leave every row one batch of four partials per thread group
+    const int ns = ma.wgs_per_head;
+    auto go = [&](auto rpw_tag) {
+        constexpr int RPW = decltype(rpw_tag)::value;
+        const int blocks = ma.Hkv * ((ma.R + RPW - 1) / RPW);
+        hipLaunchKernelGGL((merge_kernel<DT, EV, RPW>), dim3(blocks), dim3(256), 0, stream, ma);
+    };
+    if (ns <= 4 && NPG >= 8) go(std::integral_constant<int, 8>{});
+    else if (ns <= 4 * (NPG / 4)) go(std::integral_constant<int, 4>{});
+    else if (ns <= 4 * (NPG / 2)) go(std::integral_constant<int, 2>{});
+    else go(std::integral_constant<int, 1>{});
+    return hipGetLastError();
+}
+
 template <class DT>
 static hipError_t launch_merge_dt(const MergeArgs& ma, int EV, hipStream_t stream) {
-    const int blocks = ma.Hkv * ma.R;
-    if (EV == 128)
-        hipLaunchKernelGGL((merge_kernel<DT, 128>), dim3(blocks), dim3(256), 0, stream, ma);
-    else
-        hipLaunchKernelGGL((merge_kernel<DT, 64>), dim3(blocks), dim3(256), 0, stream, ma);
-    return hipGetLastError();
+    if (EV == 128) return launch_merge_ev<DT, 128>(ma, stream);
+    return launch_merge_ev<DT, 64>(ma, stream);
 }
 
 hipError_t launch_merge(const MergeArgs& ma, int dtype, int EV, hipStream_t stream) {
