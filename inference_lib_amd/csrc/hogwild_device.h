@@ -607,6 +607,85 @@ static_assert(offsetof(PagedHeader, pad) == 160, "PagedDevHeader mirrors the use
 // of the ~25-instruction integer division sequence.  d == 1 gives the multiplier 0, which stands for "n itself".
 __device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
 
+// The 40 used dwords of a PagedHeader, fetched from the kernel-argument segment with three scalar loads: requested first
+// thing in the kernel (the argument-independent setup runs while they are in flight), waited for and typed later.
+typedef int hw_i32x16 __attribute__((ext_vector_type(16)));
+typedef int hw_i32x8 __attribute__((ext_vector_type(8)));
+struct PagedHeaderBits {
+    hw_i32x16 lo, mid;
+    hw_i32x8 hi;
+};
+__device__ __forceinline__ void paged_header_request(PagedHeaderBits& hb) {
+    const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx8 %2, %3, 0x80"
+                 : "=&s"(hb.lo), "=&s"(hb.mid), "=&s"(hb.hi)
+                 : "s"(argp)
+                 : "memory");
+}
+__device__ __forceinline__ PagedDevHeader paged_header_wait(PagedHeaderBits& hb) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.mid), "+s"(hb.hi) : : "memory");
+    struct RawHeader {
+        int v[40];
+    } raw;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        raw.v[i] = hb.lo[i];
+        raw.v[16 + i] = hb.mid[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) raw.v[32 + i] = hb.hi[i];
+    return __builtin_bit_cast(PagedDevHeader, raw);
+}
+
+// Work item of a paged launch -> (worker, row group of ROWS rows within the worker, query-token range of the worker).
+// Fixed-length operator: nrg row groups per worker.  Packed queries (cu_q): row groups are numbered through the workers
+// in order, and the worker whose range contains `item` is found with a wave-wide prefix sum over 64 workers at a time;
+// found = false when the item lies beyond the last worker's row groups (the grid is sized for the worst case).
+struct PagedItem {
+    int w, rg, qs, qe;
+    bool found;
+};
+template <int ROWS>
+__device__ __forceinline__ PagedItem paged_item(const PagedDevHeader& ph, int item, int lane, int GQ) {
+    PagedItem it = {0, 0, 0, 0, false};
+    if (ph.cu_q == nullptr) {
+        it.w = fast_div(item, ph.magic_nrg);
+        it.rg = item - it.w * ph.nrg;
+        it.qs = it.w * ph.LS;
+        it.qe = it.qs + ph.LS;
+        it.found = true;
+    } else {
+        int base = 0;
+        for (int c = 0; c < ph.W && !it.found; c += 64) {
+            const int idx = c + lane;
+            const int a0 = ph.cu_q[min(idx, ph.W)], a1 = ph.cu_q[min(idx + 1, ph.W)];
+            const int cnt = idx < ph.W ? (max(a1 - a0, 0) * GQ + ROWS - 1) / ROWS : 0;
+            int inc = cnt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int v = __shfl_up(inc, off, 64);
+                if (lane >= off) inc += v;
+            }
+            const int total = __builtin_amdgcn_readlane(inc, 63);
+            if (item < base + total) {
+                const int l0 = __builtin_ctzll(__ballot(base + inc > item));
+                it.w = c + l0;
+                it.rg = item - base - __builtin_amdgcn_readlane(inc - cnt, l0);
+                it.qs = __builtin_amdgcn_readlane(a0, l0);
+                it.qe = __builtin_amdgcn_readlane(a1, l0);
+                it.found = true;
+            }
+            base += total;
+        }
+    }
+    // a malformed prefix-sum array must not lead outside the buffers
+    const int T = ph.LW * ph.LS;
+    it.qe = min(it.qe, T);
+    it.qs = min(max(it.qs, 0), it.qe);
+    return it;
+}
+
+
 // row r (0..R) of a kv head -> (worker*S + token, q head, flat q row index)
 struct RowMap {
     int ws;

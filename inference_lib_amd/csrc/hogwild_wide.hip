@@ -461,20 +461,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     const int n = lane & 15;
     const int q = lane >> 4;
 
-    typedef int i32x16 __attribute__((ext_vector_type(16)));
-    typedef int i32x8 __attribute__((ext_vector_type(8)));
-    struct HeaderBits {
-        i32x16 lo, mid;
-        i32x8 hi;
-    };
-    HeaderBits hb;
-    {
-        const auto argp = __builtin_amdgcn_kernarg_segment_ptr();
-        asm volatile("s_load_dwordx16 %0, %3, 0x0\n\ts_load_dwordx16 %1, %3, 0x40\n\ts_load_dwordx8 %2, %3, 0x80"
-                     : "=&s"(hb.lo), "=&s"(hb.mid), "=&s"(hb.hi)
-                     : "s"(argp)
-                     : "memory");
-    }
+    PagedHeaderBits hb;
+    paged_header_request(hb);
     // this wave's share of a tile's transfers: the first half of the waves fill the K image, the second half V
     const bool k_wave = wv < NW / 2;
     const int first = (k_wave ? wv : wv - NW / 2) * TPW;
@@ -498,18 +486,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.fresh = true;
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.mid), "+s"(hb.hi) : : "memory");
-    struct RawHeader {
-        int v[40];
-    } raw;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        raw.v[i] = hb.lo[i];
-        raw.v[16 + i] = hb.mid[i];
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) raw.v[32 + i] = hb.hi[i];
-    const PagedDevHeader ph = __builtin_bit_cast(PagedDevHeader, raw);
+    const PagedDevHeader ph = paged_header_wait(hb);
 
     // logical workgroup id = ((kv head * nitems) + item) * nsplit + split; consecutive ids share an XCD
     int bid = blockIdx.x;
@@ -520,42 +497,10 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     const int item = hi - hkv * ph.nitems;
     const int GQ = ph.Hq / ph.Hkv;
 
-    // item -> (worker, row group, query-token range of the worker), as in paged_attention_kernel
-    int w = 0, rg = 0, qs = 0, qe = 0;
-    if (ph.cu_q == nullptr) {
-        w = fast_div(item, ph.magic_nrg);
-        rg = item - w * ph.nrg;
-        qs = w * ph.LS;
-        qe = qs + ph.LS;
-    } else {
-        bool found = false;
-        int base = 0;
-        for (int c = 0; c < ph.W && !found; c += 64) {
-            const int idx = c + lane;
-            const int a0 = ph.cu_q[min(idx, ph.W)], a1 = ph.cu_q[min(idx + 1, ph.W)];
-            const int cnt = idx < ph.W ? (max(a1 - a0, 0) * GQ + WIDE_ROWS - 1) / WIDE_ROWS : 0;
-            int inc = cnt;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const int v = __shfl_up(inc, off, 64);
-                if (lane >= off) inc += v;
-            }
-            const int total = __builtin_amdgcn_readlane(inc, 63);
-            if (item < base + total) {
-                const int l0 = __builtin_ctzll(__ballot(base + inc > item));
-                w = c + l0;
-                rg = item - base - __builtin_amdgcn_readlane(inc - cnt, l0);
-                qs = __builtin_amdgcn_readlane(a0, l0);
-                qe = __builtin_amdgcn_readlane(a1, l0);
-                found = true;
-            }
-            base += total;
-        }
-        if (!found) return;   // the grid is sized for the worst case; uniform over the workgroup
-    }
+    const PagedItem it = paged_item<WIDE_ROWS>(ph, item, lane, GQ);
+    if (!it.found) return;                  // the grid is sized for the worst case; uniform over the workgroup
+    const int w = it.w, rg = it.rg, qs = it.qs, qe = it.qe;
     const int T = ph.LW * ph.LS;
-    qe = min(qe, T);
-    qs = min(max(qs, 0), qe);
     const int r0 = qs * GQ + rg * WIDE_ROWS;    // first row of the workgroup (global numbering: token * GQ + head in group)
     const int rend = qe * GQ;                   // end of the worker's rows
     if (r0 >= rend) return;                     // uniform over the workgroup
