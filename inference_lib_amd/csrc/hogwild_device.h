@@ -202,6 +202,10 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
 #pragma unroll
     for (int i = 0; i < G::KL; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, HW_KV_AUX);
+    // The transfers stay ahead of everything that follows in program order.  (The compiler models a transfer as a
+    // 16-byte store at its LDS base, not as the 1 KB it is, and has moved operand reads of the same slot in between the
+    // transfers of a tile on the strength of that.)
+    asm volatile("" ::: "memory");
     // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load.  Rows beyond the fragment are
     // redirected to its last row (their probabilities are zero); a tile that does not exist reads one cached line
     // (fv.idle) with every lane: loads return in order, so what such a load costs is its own latency behind the last

@@ -241,18 +241,30 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 
         // ---- stream this wave's tiles: PF buffers, the tile PF-1 steps ahead is requested right before each
         // tile is computed, so its transfer overlaps the arithmetic and the prologue above overlapped the first ----
-        for (int lt = lt0; lt < lt1; lt += PF * NWAVES) {
+        // Two loops with one instantiation of the tile arithmetic each: first the groups of PF tiles that every row of
+        // the wave sees completely, then the rest.  (With both instantiations in one loop body the compiler merges their
+        // accumulators through register copies, 48 v_mov_b64 per tile.)
+        int lt = lt0;
+        constexpr int LAST = (PF - 1) * NWAVES;     // distance of a group's last tile from its first
+        for (; maxlim > 0 && lt + LAST < lt1 && (lt + LAST + 1) * TILE <= minlim; lt += PF * NWAVES) {
+#pragma unroll
+            for (int i = 0; i < PF; ++i) {
+                const int l = lt + i * NWAVES;
+                const int nb = (i + PF - 1) % PF;   // constant after unrolling
+                const int ln = l + (PF - 1) * NWAVES;
+                load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
+                compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, l * TILE, n, q, a.sc, kslots[i]);
+            }
+        }
+        for (; lt < lt1; lt += PF * NWAVES) {
 #pragma unroll
             for (int i = 0; i < PF; ++i) {
                 const int l = lt + i * NWAVES;
                 const int t0 = l * TILE;
-                const int nb = (i + PF - 1) % PF;   // constant after unrolling
+                const int nb = (i + PF - 1) % PF;
                 const int ln = l + (PF - 1) * NWAVES;
                 load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
-                if (l < lt1 && t0 < maxlim) {
-                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
-                    else compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
-                }
+                if (l < lt1 && t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
             }
         }
         more = todo != 0;

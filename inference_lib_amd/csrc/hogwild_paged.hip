@@ -207,23 +207,35 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
             // they have arrived by the time the current tile's data has), then compute the current tile.
             TileRegs<DT, E, EV> tr[2];
             issue_tile(tr[0], kslots[0], bt_a, gw);
-            for (int t = gw; t * TILE < maxlim; t += 2 * NW) {
+            // Two loops with one instantiation of the tile arithmetic each (see attention_kernel): pairs of tiles every
+            // row of the wave sees completely, then the rest.
+            int t = gw;
+            for (; (t + NW + 1) * TILE <= minlim; t += 2 * NW) {
                 {
                     const int bt_n = bt_load(t + 2 * NW);
                     issue_tile(tr[1], kslots[1], bt_b, t + NW);
-                    const int t0 = t * TILE;
-                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
-                    else compute_tile<DT, E, EV, RB, true, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
+                    compute_tile<DT, E, EV, RB, false, QREG>(tr[0], q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, kslots[0]);
+                    bt_a = bt_n;
+                }
+                {
+                    const int bt_n = bt_load(t + 3 * NW);
+                    issue_tile(tr[0], kslots[0], bt_a, t + 2 * NW);
+                    compute_tile<DT, E, EV, RB, false, QREG>(tr[1], q_lds, qreg, lim, st, (t + NW) * TILE, n, q, ph.sc, kslots[1]);
+                    bt_b = bt_n;
+                }
+            }
+            for (; t * TILE < maxlim; t += 2 * NW) {
+                {
+                    const int bt_n = bt_load(t + 2 * NW);
+                    issue_tile(tr[1], kslots[1], bt_b, t + NW);
+                    compute_tile<DT, E, EV, RB, true, QREG>(tr[0], q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, kslots[0]);
                     bt_a = bt_n;
                 }
                 {
                     const int bt_n = bt_load(t + 3 * NW);
                     issue_tile(tr[0], kslots[0], bt_a, t + 2 * NW);
                     const int t0 = (t + NW) * TILE;
-                    if (t0 < maxlim) {
-                        if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
-                        else compute_tile<DT, E, EV, RB, true, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
-                    }
+                    if (t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
                     bt_b = bt_n;
                 }
             }

@@ -332,29 +332,39 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
 #pragma unroll
         for (int i = 1; i < D; ++i) request(i, lt0 + i);
 
-        bool done = false;
-        for (int lt = lt0; !done; lt += NS) {
-#pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                const int l = lt + i;
-                if (l >= lt1) {          // uniform over the workgroup: every wave leaves at the same tile
-                    done = true;
-                    break;
-                }
-                request((i + D) % NS, l + D);
-                // Wait for this wave's own transfers of tile l, then meet the other waves: tile l is complete in LDS.  The
-                // D requests issued since are the only newer memory operations that may stay outstanding (loads complete
-                // in order; stores still in flight only make the wait longer).  A plain barrier, not __syncthreads(): its
-                // release fence would wait for every outstanding transfer, the look-ahead included.
+        {
+            // Two loops, one instantiation of the tile arithmetic in each: first the tiles every row of this wave sees
+            // completely, then the rest.  With both instantiations in one loop body the compiler merges their accumulators
+            // through copies (48 v_mov_b64 per tile).  The waves of a workgroup may change loops at different tiles; each
+            // still passes one barrier per tile.
+            int sl = 0;                                   // ring slot of tile l
+            int l = lt0;
+            auto arrive = [&]() {                         // request tile l + D, wait for tile l
+                int rs = sl + D;
+                if (rs >= NS) rs -= NS;
+                request(rs, l + D);
                 asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
-                const int t0 = l * TILE;
-                if (t0 < maxlim) {
-                    const char* slot = ring + i * SLOT;
+            };
+            const int lfast = maxlim > 0 ? min(lt1, minlim / TILE) : lt0;
+#pragma unroll 1
+            for (; l < lfast; ++l) {
+                arrive();
+                const char* slot = ring + sl * SLOT;
+                TileRegs<DT, E, EV> tr;
+                read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
+                compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot);
+                sl = sl + 1 == NS ? 0 : sl + 1;
+            }
+#pragma unroll 1
+            for (; l < lt1; ++l) {
+                arrive();
+                if (l * TILE < maxlim) {
+                    const char* slot = ring + sl * SLOT;
                     TileRegs<DT, E, EV> tr;
                     read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
-                    if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, slot);
-                    else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, a.sc, slot);
+                    compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot);
                 }
+                sl = sl + 1 == NS ? 0 : sl + 1;
             }
         }
         // the requests behind the last tile (they fetched nothing) must have landed before the ring is used again
@@ -608,29 +618,38 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
                 request(i, src);
             }
             addresses(src, split + D * ns);
-            bool done = false;
-            for (int k0 = 0; !done; k0 += NS) {
-#pragma unroll
-                for (int i = 0; i < NS; ++i) {
-                    const int t = split + (k0 + i) * ns;
-                    if (t * TILE >= wgmax) {      // uniform over the workgroup: every wave leaves at the same tile
-                        done = true;
-                        break;
-                    }
-                    request((i + D) % NS, src);   // tile t + D * ns
-                    // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
-                    // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
-                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
-                    addresses(src, t + (D + 1) * ns);
-                    const int t0 = t * TILE;
-                    if (t0 < maxlim) {
-                        const char* slot = ring + i * SLOT;
-                        TileRegs<DT, E, EV> tr;
-                        read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
-                        if (t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t0, n, q, ph.sc, slot);
-                        else compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t0, n, q, ph.sc, slot);
-                    }
+            // two loops with one instantiation of the tile arithmetic each (see attention_wide_kernel)
+            int sl = 0;
+            int t = split;
+            auto arrive = [&]() {                         // request tile t + D * ns, wait for tile t, form the next addresses
+                int rs = sl + D;
+                if (rs >= NS) rs -= NS;
+                request(rs, src);
+                // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
+                // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
+                addresses(src, t + (D + 1) * ns);
+            };
+            const int tfast = maxlim > 0 ? min(minlim, wgmax) / TILE : 0;   // tiles below it are seen completely by every row of the wave
+#pragma unroll 1
+            for (; t < tfast; t += ns) {
+                arrive();
+                const char* slot = ring + sl * SLOT;
+                TileRegs<DT, E, EV> tr;
+                read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
+                compute_tile<DT, E, EV, RB, false, true>(tr, q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot);
+                sl = sl + 1 == NS ? 0 : sl + 1;
+            }
+#pragma unroll 1
+            for (; t * TILE < wgmax; t += ns) {           // uniform over the workgroup: every wave leaves at the same tile
+                arrive();
+                if (t * TILE < maxlim) {
+                    const char* slot = ring + sl * SLOT;
+                    TileRegs<DT, E, EV> tr;
+                    read_v_rows<DT, E, EV>(slot + KBYTES, n, q, tr);
+                    compute_tile<DT, E, EV, RB, true, true>(tr, q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot);
                 }
+                sl = sl + 1 == NS ? 0 : sl + 1;
             }
             // the requests behind the last tile must have landed before the ring is used again
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
