@@ -266,10 +266,15 @@ struct WaveState {
 // One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
 // VS = the logits S^T = K Q^T are formed with VALU dot products (v_dot2 / v_fma) instead of MFMA, in the same lane
 // layout (row = lane % 16, eight tokens per lane): the measured alternative for workloads with few query rows.
-template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false>
-__device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
-                                             WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage) {
+// VLDS = the V rows of the tile lie in LDS as a row-major image at `vimg` (the kernels whose waves share every tile) and
+// are read here, after the K operands: LDS answers in order, and the logits wait for K only.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false>
+__device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
+                                             WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage,
+                                             const char* vimg = nullptr) {
     typedef Geo<DT, E, EV> G;
+    TileRegs<DT, E, EV> t_own;
+    const TileRegs<DT, E, EV>& t = VLDS ? t_own : t_in;
 #ifdef HW_NO_COMPUTE   // tuning aid: consume the tile without doing the arithmetic
     {
         u32 x = 0;
@@ -306,6 +311,22 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t, const
                 sacc[rb][idx >> 2][idx & 3] = acc;
             }
         }
+    } else if constexpr (VLDS) {
+        u32x4 kop[2][G::KJ];
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int j = 0; j < G::KJ; ++j) kop[tb][j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
+        read_v_rows<DT, E, EV>(vimg, n, q, t_own);
+#pragma unroll
+        for (int tb = 0; tb < 2; ++tb)
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[tb][j], qreg[rb * G::KJ + j], acc);
+                sacc[rb][tb] = acc;
+            }
     } else
 #pragma unroll
     for (int tb = 0; tb < 2; ++tb) {
