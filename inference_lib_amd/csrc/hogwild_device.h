@@ -100,12 +100,19 @@ __device__ __forceinline__ void quarter_pairs(float v, int step, float& a, float
         b = __uint_as_float(r[1]);
     }
 }
+// max of two values that are never NaN.  fmaxf() on the halves of a lane exchange makes the compiler canonicalise both
+// inputs first (v_max_f32 x, x, x: two extra instructions per maximum, 8 per tile); the instruction itself needs none.
+__device__ __forceinline__ float max_nn(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
 __device__ __forceinline__ float quarter_max(float v) {
     float a, b;
     quarter_pairs(v, 32, a, b);
-    v = fmaxf(a, b);
+    v = max_nn(a, b);
     quarter_pairs(v, 16, a, b);
-    return fmaxf(a, b);
+    return max_nn(a, b);
 }
 __device__ __forceinline__ float quarter_sum(float v) {
     float a, b;
@@ -254,6 +261,28 @@ __device__ __forceinline__ void read_v_rows(const char* vimg, int n, int q, Tile
     }
 }
 
+// V image for transposed reads (the kernels whose waves share every tile, 16-bit types): rows of VROW bytes, the 32-byte
+// segments of a row (16 elements: what one MFMA block of outputs needs) stored at segment ^ (row & 3), so that the four
+// consecutive rows one 16-lane group reads lie in different banks.  In units of 16-byte chunks the key is 2 (row & 3).
+__device__ __forceinline__ int vimg_chunk_key(int row) { return (row & 3) << 1; }
+
+typedef short v4i16 __attribute__((ext_vector_type(4)));
+// ds_read_b64_tr_b16: within a 16-lane group, lanes 4r .. 4r+3 name the four 8-byte pieces of row r (r = 0..3, 16
+// elements), and lane d receives element d of rows 0..3: a 4 x 16 block delivered by columns, which is the MFMA operand
+// layout of V^T (lane = output element, four consecutive tokens per read) without any register shuffling.
+__device__ __forceinline__ u32x2 lds_read_tr16(const char* p) {
+    const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(p));
+    return __builtin_bit_cast(u32x2, r);
+}
+// Per-lane byte offsets into a swizzled V image for output block c (16 elements) of the lane's quarter-wave: entry m
+// serves the blocks with c % 4 == m; add (c / 4) * 128 for the block and 16 * VROW for the tile's second 16 tokens.
+template <int VROW>
+__device__ __forceinline__ void vtr_lane_offsets(unsigned (&voff)[4], int lane) {
+    const int q = lane >> 4, r = (lane >> 2) & 3, j = lane & 3;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) voff[m] = (unsigned)((q * 4 + r) * VROW + ((m ^ r) << 5) + 8 * j);
+}
+
 // Running state of one wave: RB row blocks of 16 rows each.
 template <int RB, int NOC>
 struct WaveState {
@@ -268,10 +297,12 @@ struct WaveState {
 // layout (row = lane % 16, eight tokens per lane): the measured alternative for workloads with few query rows.
 // VLDS = the V rows of the tile lie in LDS as a row-major image at `vimg` (the kernels whose waves share every tile) and
 // are read here, after the K operands: LDS answers in order, and the logits wait for K only.
-template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false>
+// VTR = the V image is swizzled for transposed reads (vimg_chunk_key) and the V^T operands come straight out of it
+// (lds_read_tr16, per-lane offsets `voff` from vtr_lane_offsets); output block c then holds elements 16c .. 16c+15.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false, bool VTR = false>
 __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
                                              WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage,
-                                             const char* vimg = nullptr) {
+                                             const char* vimg = nullptr, const unsigned* voff = nullptr) {
     typedef Geo<DT, E, EV> G;
     TileRegs<DT, E, EV> t_own;
     const TileRegs<DT, E, EV>& t = VLDS ? t_own : t_in;
@@ -317,7 +348,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
             for (int j = 0; j < G::KJ; ++j) kop[tb][j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
-        read_v_rows<DT, E, EV>(vimg, n, q, t_own);
+        if constexpr (!VTR) read_v_rows<DT, E, EV>(vimg, n, q, t_own);
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
@@ -372,7 +403,8 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             mx = fmaxf(mx, s[rb][idx]);
         }
         mx = quarter_max(mx);
-        mxs[rb] = mx < -1.0e29f ? NEG_BIG : mx * sc;      // sc > 0: scaling commutes with the max; nothing visible stays NEG_BIG
+        // sc > 0: scaling commutes with the max; a row that sees nothing of a masked tile keeps NEG_BIG
+        mxs[rb] = MASKED ? (mx < -1.0e29f ? NEG_BIG : mx * sc) : mx * sc;
         need = need || (mxs[rb] > st.m[rb] + LAZY_LOG2);
     }
     if (__builtin_amdgcn_ballot_w64(need) != 0) {        // uniform over the wave
@@ -394,11 +426,11 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
     for (int rb = 0; rb < RB; ++rb) {
         // a row that has seen nothing yet keeps the reference NEG_BIG; exponentiate against 0 so its masked slots give 0
         const float mref = MASKED ? (st.m[rb] < -1.0e29f ? 0.f : st.m[rb]) : st.m[rb];
-        float psum = 0.f;
+        float psum;
 #pragma unroll
         for (int idx = 0; idx < 8; ++idx) {
             p[rb][idx] = fast_exp2(__builtin_fmaf(s[rb][idx], sc, -mref));
-            psum += p[rb][idx];
+            psum = idx == 0 ? p[rb][0] : psum + p[rb][idx];
         }
         st.l[rb] += psum;
     }
@@ -412,6 +444,16 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             pp[rb].z = Elem<DT>::pack2(p[rb][4], p[rb][5]);
             pp[rb].w = Elem<DT>::pack2(p[rb][6], p[rb][7]);
         }
+        if constexpr (VTR) {
+#pragma unroll
+            for (int c = 0; c < G::NOC; ++c) {
+                const char* vp = vimg + voff[c & 3] + (c >> 2) * 128;
+                const u32x2 a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
+                const u32x4 vop = {a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) st.o[rb][c] = Elem<DT>::mfma(vop, pp[rb], st.o[rb][c]);
+            }
+        } else
         // dword d of a lane's V row holds ev (n*EVL + 2d, n*EVL + 2d + 1); gather the 8 tokens of each ev.
 #pragma unroll
         for (int d = 0; d < G::VW; ++d) {

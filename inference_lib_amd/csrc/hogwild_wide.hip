@@ -212,7 +212,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         const int p = (first + j) * 64 + lane;
         const int row = p / G::CPR, slot = p % G::CPR;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
-        off[j] = k_wave ? row * G::KROW + ((slot ^ key) << 4) : p * 16;
+        off[j] = k_wave ? row * G::KROW + ((slot ^ key) << 4) : row * G::VROW + ((slot ^ vimg_chunk_key(row)) << 4);
     }
     const unsigned long long my_image_ptr = k_wave ? my_k : my_v;   // lane f: this wave's image of fragment f
     const int image_row = k_wave ? G::KROW : G::VROW;               // bytes per token in it
@@ -226,6 +226,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.fresh = true;
+    unsigned voff[4];                             // this lane's positions in a V image (transposed reads)
+    vtr_lane_offsets<G::VROW>(voff, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
 
@@ -350,7 +352,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
             for (; l < lfast; ++l) {
                 arrive();
                 const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES);
+                compute_tile<DT, E, EV, RB, false, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
 #pragma unroll 1
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
                 arrive();
                 if (l * TILE < maxlim) {
                     const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES);
+                    compute_tile<DT, E, EV, RB, true, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
                 }
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
@@ -387,11 +389,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
             const int row0 = w0 + rb * 16;                            // first row of the block
             const size_t prow0 = (size_t)(hkv * a.wgs_per_head + g) * a.R + row0;
 #pragma unroll
-            for (int c0 = 0; c0 < G::NOC; c0 += 4)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    *reinterpret_cast<f32x4*>(stage + n * OSTR + out_ev<DT, EV>(c0, 4 * q + i)) =
-                        f32x4{st.o[rb][c0][i], st.o[rb][c0 + 1][i], st.o[rb][c0 + 2][i], st.o[rb][c0 + 3][i]};
+            for (int c = 0; c < G::NOC; ++c)              // block c, accumulator rows 4q .. 4q+3 = elements 16c + 4q ..
+                *reinterpret_cast<f32x4*>(stage + n * OSTR + 16 * c + 4 * q) = st.o[rb][c];
             if (q == 0 && row0 + n < a.R) *reinterpret_cast<HW_GLOBAL f32x2*>(a.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
             // (one wave: the LDS writes above are complete before the reads below are issued, in program order, and
             // the reads before the next block's writes)
@@ -480,7 +479,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         const int row = (first + j) * RPL + lrow;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
         trow[j] = row;
-        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : lslot) << 4);
+        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : (lslot ^ vimg_chunk_key(row))) << 4);
     }
     const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
     WaveState<RB, G::NOC> st;
@@ -492,6 +491,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.fresh = true;
+    unsigned voff[4];                             // this lane's positions in a V image (transposed reads)
+    vtr_lane_offsets<G::VROW>(voff, lane);
     const PagedDevHeader ph = paged_header_wait(hb);
 
     // logical workgroup id = ((kv head * nitems) + item) * nsplit + split; consecutive ids share an XCD
@@ -631,7 +632,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
             for (; t < tfast; t += ns) {
                 arrive();
                 const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES);
+                compute_tile<DT, E, EV, RB, false, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
 #pragma unroll 1
@@ -639,7 +640,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
                 arrive();
                 if (t * TILE < maxlim) {
                     const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES);
+                    compute_tile<DT, E, EV, RB, true, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                 }
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
@@ -660,11 +661,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
             const int row0 = w0 + rb * 16;
             const size_t prow0 = (size_t)(hkv * ph.nsplit + split) * ph.R + row0;
 #pragma unroll
-            for (int c0 = 0; c0 < G::NOC; c0 += 4)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    *reinterpret_cast<f32x4*>(stage + n * OSTR + out_ev<DT, EV>(c0, 4 * q + i)) =
-                        f32x4{st.o[rb][c0][i], st.o[rb][c0 + 1][i], st.o[rb][c0 + 2][i], st.o[rb][c0 + 3][i]};
+            for (int c = 0; c < G::NOC; ++c)              // block c, accumulator rows 4q .. 4q+3 = elements 16c + 4q ..
+                *reinterpret_cast<f32x4*>(stage + n * OSTR + 16 * c + 4 * q) = st.o[rb][c];
             if (q == 0 && row0 + n < rend) *reinterpret_cast<HW_GLOBAL f32x2*>(ph.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
             const int nvalid = min(16, rend - row0);
             HW_GLOBAL float* dst = ph.part_o + prow0 * EV;
