@@ -243,9 +243,11 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
         // tile is computed, so its transfer overlaps the arithmetic and the prologue above overlapped the first ----
         // Two loops with one instantiation of the tile arithmetic each: first the groups of PF tiles that every row of
         // the wave sees completely, then the rest.  (With both instantiations in one loop body the compiler merges their
-        // accumulators through register copies, 48 v_mov_b64 per tile.)
+        // accumulators through register copies, 48 v_mov_b64 per tile.)  The fp32 kernels keep the one loop with both: their
+        // tiles are MFMA time, and the second loop cost them 0.45 us per launch on the small workloads they serve.
         int lt = lt0;
         constexpr int LAST = (PF - 1) * NWAVES;     // distance of a group's last tile from its first
+        if constexpr (G::SZ != 4)
         for (; maxlim > 0 && lt + LAST < lt1 && (lt + LAST + 1) * TILE <= minlim; lt += PF * NWAVES) {
 #pragma unroll
             for (int i = 0; i < PF; ++i) {
@@ -264,7 +266,9 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
                 const int nb = (i + PF - 1) % PF;
                 const int ln = l + (PF - 1) * NWAVES;
                 load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
-                if (l < lt1 && t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                const bool live = l < lt1 && t0 < maxlim;
+                if (G::SZ == 4 && live && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
+                else if (live) compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
             }
         }
         more = todo != 0;

@@ -210,6 +210,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
             // Two loops with one instantiation of the tile arithmetic each (see attention_kernel): pairs of tiles every
             // row of the wave sees completely, then the rest.
             int t = gw;
+            if constexpr (G::SZ != 4)               // (the fp32 kernels keep one loop with both instantiations, see attention_kernel)
             for (; (t + NW + 1) * TILE <= minlim; t += 2 * NW) {
                 {
                     const int bt_n = bt_load(t + 2 * NW);
@@ -228,14 +229,17 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
                 {
                     const int bt_n = bt_load(t + 2 * NW);
                     issue_tile(tr[1], kslots[1], bt_b, t + NW);
-                    compute_tile<DT, E, EV, RB, true, QREG>(tr[0], q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, kslots[0]);
+                    const int t0 = t * TILE;
+                    if (G::SZ == 4 && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
+                    else compute_tile<DT, E, EV, RB, true, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
                     bt_a = bt_n;
                 }
                 {
                     const int bt_n = bt_load(t + 3 * NW);
                     issue_tile(tr[0], kslots[0], bt_a, t + 2 * NW);
                     const int t0 = (t + NW) * TILE;
-                    if (t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
+                    if (G::SZ == 4 && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
+                    else if (t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
                     bt_b = bt_n;
                 }
             }
