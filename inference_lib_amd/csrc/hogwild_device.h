@@ -262,9 +262,15 @@ __device__ __forceinline__ void read_v_rows(const char* vimg, int n, int q, Tile
 }
 
 // V image for transposed reads (the kernels whose waves share every tile, 16-bit types): rows of VROW bytes, the 32-byte
-// segments of a row (16 elements: what one MFMA block of outputs needs) stored at segment ^ (row & 3), so that the four
-// consecutive rows one 16-lane group reads lie in different banks.  In units of 16-byte chunks the key is 2 (row & 3).
-__device__ __forceinline__ int vimg_chunk_key(int row) { return (row & 3) << 1; }
+// segments of a row (16 elements: what one MFMA block of outputs needs) stored at segment ^ key(row), the key chosen so
+// that the eight consecutive rows two neighbouring 16-lane groups read (2 x 4 rows x 32 bytes) cover all 64 banks:
+// rows of 256 bytes start at bank 0, so the key is row & 7; rows of 128 bytes alternate between the two halves of the
+// banks by themselves and the key is (row >> 1) & 3.
+template <int VROW>
+__device__ __forceinline__ int vimg_segment_key(int row) {
+    static_assert(VROW == 256 || VROW == 128, "head dims 128 and 64 in 16-bit types");
+    return VROW == 256 ? (row & 7) : ((row >> 1) & 3);
+}
 
 typedef short v4i16 __attribute__((ext_vector_type(4)));
 // ds_read_b64_tr_b16: within a 16-lane group, lanes 4r .. 4r+3 name the four 8-byte pieces of row r (r = 0..3, 16
@@ -274,13 +280,14 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char* p) {
     const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(p));
     return __builtin_bit_cast(u32x2, r);
 }
-// Per-lane byte offsets into a swizzled V image for output block c (16 elements) of the lane's quarter-wave: entry m
-// serves the blocks with c % 4 == m; add (c / 4) * 128 for the block and 16 * VROW for the tile's second 16 tokens.
+// Per-lane byte offsets into a swizzled V image for output block c (16 elements) and the first 16 tokens of a tile (the
+// lane names row 4q + r, r = (lane / 4) % 4, piece lane % 4); add 16 * VROW for the second 16 tokens (same key).
 template <int VROW>
-__device__ __forceinline__ void vtr_lane_offsets(unsigned (&voff)[4], int lane) {
+__device__ __forceinline__ void vtr_lane_offsets(unsigned (&voff)[VROW / 32], int lane) {
     const int q = lane >> 4, r = (lane >> 2) & 3, j = lane & 3;
+    const int row = q * 4 + r;
 #pragma unroll
-    for (int m = 0; m < 4; ++m) voff[m] = (unsigned)((q * 4 + r) * VROW + ((m ^ r) << 5) + 8 * j);
+    for (int c = 0; c < VROW / 32; ++c) voff[c] = (unsigned)(row * VROW + ((c ^ vimg_segment_key<VROW>(row)) << 5) + 8 * j);
 }
 
 // Running state of one wave: RB row blocks of 16 rows each.
@@ -447,7 +454,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
         if constexpr (VTR) {
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c) {
-                const char* vp = vimg + voff[c & 3] + (c >> 2) * 128;
+                const char* vp = vimg + voff[c];
                 const u32x2 a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
                 const u32x4 vop = {a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
 #pragma unroll

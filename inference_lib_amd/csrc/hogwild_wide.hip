@@ -212,7 +212,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         const int p = (first + j) * 64 + lane;
         const int row = p / G::CPR, slot = p % G::CPR;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
-        off[j] = k_wave ? row * G::KROW + ((slot ^ key) << 4) : row * G::VROW + ((slot ^ vimg_chunk_key(row)) << 4);
+        off[j] = k_wave ? row * G::KROW + ((slot ^ key) << 4) : row * G::VROW + ((slot ^ (2 * vimg_segment_key<G::VROW>(row))) << 4);
     }
     const unsigned long long my_image_ptr = k_wave ? my_k : my_v;   // lane f: this wave's image of fragment f
     const int image_row = k_wave ? G::KROW : G::VROW;               // bytes per token in it
@@ -226,7 +226,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.fresh = true;
-    unsigned voff[4];                             // this lane's positions in a V image (transposed reads)
+    unsigned voff[G::NOC];                             // this lane's positions in a V image (transposed reads)
     vtr_lane_offsets<G::VROW>(voff, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
@@ -298,7 +298,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
         if (!PRE && staged) {
             wrot.stage(cs_lds, tid, nws);
-            __syncthreads();
+            // The barrier above has waited for every load of open_segment: the other look-ahead tiles can be requested
+            // here, ahead of the rotation arithmetic, which waits for nothing from memory any more.  (An LDS-only barrier
+            // again: __syncthreads() would wait for the requests just issued.)
+#pragma unroll
+            for (int i = 1; i < D; ++i) request(i, lt0 + i);
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
             wrot.rotate(a, q_lds, cs_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid, ws_lo);
         } else {
             qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
@@ -331,8 +336,10 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         }
         maxlim = __builtin_amdgcn_readfirstlane(maxlim);
         minlim = __builtin_amdgcn_readfirstlane(minlim);
+        if (PRE || !staged) {
 #pragma unroll
-        for (int i = 1; i < D; ++i) request(i, lt0 + i);
+            for (int i = 1; i < D; ++i) request(i, lt0 + i);
+        }
 
         {
             // Two loops, one instantiation of the tile arithmetic in each: first the tiles every row of this wave sees
@@ -479,7 +486,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         const int row = (first + j) * RPL + lrow;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
         trow[j] = row;
-        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : (lslot ^ vimg_chunk_key(row))) << 4);
+        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : (lslot ^ (2 * vimg_segment_key<G::VROW>(row)))) << 4);
     }
     const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
     WaveState<RB, G::NOC> st;
@@ -491,7 +498,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
     st.fresh = true;
-    unsigned voff[4];                             // this lane's positions in a V image (transposed reads)
+    unsigned voff[G::NOC];                             // this lane's positions in a V image (transposed reads)
     vtr_lane_offsets<G::VROW>(voff, lane);
     const PagedDevHeader ph = paged_header_wait(hb);
 
