@@ -296,3 +296,30 @@ def test_wide_kernel_split_invariance_and_refusals():
                  sines=c32.sin, row_blocks=8).run()
     torch.cuda.synchronize()
     assert torch.isfinite(out32).all()
+
+
+@pytest.mark.parametrize("row_blocks", [8, 2])
+@pytest.mark.parametrize("dtype,E", [("bf16", 128), ("f16", 64)])
+def test_waves_leave_the_unmasked_tiles_at_different_places(oracle, row_blocks, dtype, E):
+    """The tile loop is two loops (tiles every row of a wave sees completely, then the rest).  Here the rows of one
+    workgroup see different amounts of every fragment, so its waves change loops at different tiles: bounds exactly on a
+    tile boundary, one token beyond it, nothing at all, one token, everything, per worker and per fragment."""
+    from inference_lib_amd import cases
+    W, S, Hq, Hkv = 8, 4, 8, 2                     # 128 rows per kv head; a wave of the 128-row kernel owns two workers
+    lens = (200, 96, 33, 64, 40, 17, 128, 31, 70)  # prompt + one segment per worker
+    c = cases.small_case(dtype=dtype, W=W, S=S, Hq=Hq, Hkv=Hkv, E=E, lens=lens, seed=21)
+    loc = c.locations.clone()                      # [F, W, S]: a row sees positions <= its location
+    for f, L in enumerate(lens):
+        marks = [0, 1, 31, 32, 33, 64, L - 1, L]   # visible tokens of the fragment: tile boundaries and their neighbours
+        for w in range(W):
+            seen = min(marks[(3 * f + w) % 8], L)
+            for s in range(S):
+                loc[f, w, s] = min(seen + (s % 2), L) - 1      # the tokens of a worker differ by one
+    c.locations = loc
+    c.cos, c.sin = cases.rope_tables(loc, E, 1e4)
+    print(f"{dtype} E={E} row_blocks={row_blocks} lens={lens}", flush=True)
+    want_o, want_l, want_rq = oracle_fused(oracle, c)
+    out, lse, rq = run_fused(c.to(_dev()), row_blocks=row_blocks)
+    assert_close("out", out, want_o, TOL[dtype])
+    assert_close("lse", lse, want_l, TOL[dtype])
+    assert_close("rq", rq, want_rq, 3.2e-2)
