@@ -77,7 +77,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     // transfers does not extend to the other slots.  Kernels that run one workgroup per CU have LDS to spare and give
     // the epilogue exchange memory of its own, so that a wave can hand over its accumulators the moment it is done; in
     // the others the exchange reuses the memory of slot 0.
-    constexpr bool EXSEP = MINW == 1 && sizeof(Ex) + (PF > 1 ? 2 : 1) * SBYTES + ROWS * G::QSTR + 1024 <= 160 * 1024;
+    constexpr bool EXSEP = MINW == 1 && sizeof(Ex) + PF * SBYTES + ROWS * G::QSTR + 1024 <= 160 * 1024;
     union Slot0 {
         char k[SBYTES];
         char ex[EXSEP ? 16 : sizeof(Ex)];
