@@ -238,29 +238,6 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
     }
 }
 
-// The V rows of a tile that lies complete in LDS, row-major (VROW bytes per token), in the layout of TileRegs (the
-// kernel whose waves share every tile).
-template <class DT, int E, int EV>
-__device__ __forceinline__ void read_v_rows(const char* vimg, int n, int q, TileRegs<DT, E, EV>& t) {
-    typedef Geo<DT, E, EV> G;
-#pragma unroll
-    for (int idx = 0; idx < 8; ++idx) {
-        const char* vp = vimg + slot_token(q, idx) * G::VROW + n * (G::VW * 4);   // lane n: VW dwords of the row
-        if constexpr (G::VW == 4) {
-            const u32x4 x = *reinterpret_cast<const u32x4*>(vp);
-            t.v[idx][0] = x.x;
-            t.v[idx][1] = x.y;
-            t.v[idx][2] = x.z;
-            t.v[idx][3] = x.w;
-        } else {
-            static_assert(G::VW == 2, "head dims 64 and 128");
-            const u32x2 x = *reinterpret_cast<const u32x2*>(vp);
-            t.v[idx][0] = x.x;
-            t.v[idx][1] = x.y;
-        }
-    }
-}
-
 // V image for transposed reads (the kernels whose waves share every tile, 16-bit types): rows of VROW bytes, the 32-byte
 // segments of a row (16 elements: what one MFMA block of outputs needs) stored at segment ^ key(row), the key chosen so
 // that the eight consecutive rows two neighbouring 16-lane groups read (2 x 4 rows x 32 bytes) cover all 64 banks:
@@ -302,17 +279,16 @@ struct WaveState {
 // One 32-token tile against all rows.  MASKED = false is the fast path for tiles every row sees completely.
 // VS = the logits S^T = K Q^T are formed with VALU dot products (v_dot2 / v_fma) instead of MFMA, in the same lane
 // layout (row = lane % 16, eight tokens per lane): the measured alternative for workloads with few query rows.
-// VLDS = the V rows of the tile lie in LDS as a row-major image at `vimg` (the kernels whose waves share every tile) and
-// are read here, after the K operands: LDS answers in order, and the logits wait for K only.
-// VTR = the V image is swizzled for transposed reads (vimg_chunk_key) and the V^T operands come straight out of it
-// (lds_read_tr16, per-lane offsets `voff` from vtr_lane_offsets); output block c then holds elements 16c .. 16c+15.
-template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false, bool VTR = false>
+// VLDS = the V rows of the tile lie in LDS as an image at `vimg`, swizzled for transposed reads (vimg_segment_key; the
+// kernels whose waves share every tile, 16-bit types): the K operands are read first (LDS answers in order, and the
+// logits wait for K only), the V^T operands come straight out of the image (lds_read_tr16, per-lane offsets `voff` from
+// vtr_lane_offsets), and output block c then holds elements 16c .. 16c+15.  `t_in` is not used.
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false>
 __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
                                              WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage,
                                              const char* vimg = nullptr, const unsigned* voff = nullptr) {
     typedef Geo<DT, E, EV> G;
-    TileRegs<DT, E, EV> t_own;
-    const TileRegs<DT, E, EV>& t = VLDS ? t_own : t_in;
+    const TileRegs<DT, E, EV>& t = t_in;
 #ifdef HW_NO_COMPUTE   // tuning aid: consume the tile without doing the arithmetic
     {
         u32 x = 0;
@@ -355,7 +331,6 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
             for (int j = 0; j < G::KJ; ++j) kop[tb][j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
-        if constexpr (!VTR) read_v_rows<DT, E, EV>(vimg, n, q, t_own);
 #pragma unroll
         for (int tb = 0; tb < 2; ++tb)
 #pragma unroll
@@ -451,7 +426,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             pp[rb].z = Elem<DT>::pack2(p[rb][4], p[rb][5]);
             pp[rb].w = Elem<DT>::pack2(p[rb][6], p[rb][7]);
         }
-        if constexpr (VTR) {
+        if constexpr (VLDS) {
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c) {
                 const char* vp = vimg + voff[c];

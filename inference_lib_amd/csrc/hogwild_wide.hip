@@ -359,7 +359,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
             for (; l < lfast; ++l) {
                 arrive();
                 const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
+                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
 #pragma unroll 1
@@ -367,7 +367,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
                 arrive();
                 if (l * TILE < maxlim) {
                     const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
+                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
                 }
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
@@ -639,7 +639,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
             for (; t < tfast; t += ns) {
                 arrive();
                 const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
 #pragma unroll 1
@@ -647,7 +647,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
                 arrive();
                 if (t * TILE < maxlim) {
                     const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                 }
                 sl = sl + 1 == NS ? 0 : sl + 1;
             }
