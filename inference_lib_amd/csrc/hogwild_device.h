@@ -206,12 +206,13 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
                                           int n, int q, bool real) {
     typedef Geo<DT, E, EV> G;
     const unsigned kb = real ? (unsigned)(t0 * G::KROW) : OOB_OFFSET;
+    // The transfers keep their place in program order: behind every earlier read of the slot and ahead of everything
+    // that follows.  (The compiler models a transfer as a 16-byte store at its LDS base, not as the 1 KB it is, and has
+    // moved operand reads of the same slot in between the transfers of a tile on the strength of that.)
+    asm volatile("" ::: "memory");
 #pragma unroll
     for (int i = 0; i < G::KL; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(fv.k, HW_LDS_PTR(kslot + i * 1024), 16, kb + koff[i], 0, 0, HW_KV_AUX);
-    // The transfers stay ahead of everything that follows in program order.  (The compiler models a transfer as a
-    // 16-byte store at its LDS base, not as the 1 KB it is, and has moved operand reads of the same slot in between the
-    // transfers of a tile on the strength of that.)
     asm volatile("" ::: "memory");
     // V: a quarter-wave reads one whole row (or half of a 512-byte row) per load.  Rows beyond the fragment are
     // redirected to its last row (their probabilities are zero); a tile that does not exist reads one cached line

@@ -172,12 +172,14 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
             const int jstar = min(max(maxlim - 1 - t * TILE, 0), 31);
             const int rstar = __builtin_amdgcn_readlane(rid, jstar);
             rid = tok_raw < maxlim ? rid : rstar;
+            asm volatile("" ::: "memory");   // the transfers keep their place between the reads of the slot (see load_tile)
 #pragma unroll
             for (int i = 0; i < G::KL; ++i) {
                 const int r = __shfl(rid, i * RPL + lrow, 64);
                 const HW_GLOBAL char* src = ph.kcache + (unsigned long long)(unsigned)r * G::KROW + k_chunk(i);
                 __builtin_amdgcn_global_load_lds(src, HW_LDS_PTR(kslot + i * 1024), 16, 0, HW_KV_AUX);
             }
+            asm volatile("" ::: "memory");
 #pragma unroll
             for (int idx = 0; idx < 8; ++idx) {
                 const int r = __shfl(rid, slot_token(q, idx), 64);
