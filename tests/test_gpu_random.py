@@ -155,3 +155,20 @@ def test_fused_random_shapes_with_device_lengths(oracle, seed):
     assert_close("out", out, want_o, tol)
     assert_close("lse", lse, want_l, tol)
     assert_close("rq", rq, want_rq, 1e-5 if c.dtype == "f32" else 3.2e-2)
+
+
+def test_extended_sweep(oracle):
+    """Opt-in: the five generators above over a seed range given as HOGWILD_SWEEP_SEEDS=lo:hi (e.g. 100:4000, about nine
+    minutes on one GPU); skipped when the variable is not set.  The seed and generator are printed before each case."""
+    import os
+    spec = os.environ.get("HOGWILD_SWEEP_SEEDS")
+    if not spec:
+        pytest.skip("set HOGWILD_SWEEP_SEEDS=lo:hi to run the extended sweep")
+    lo, hi = (int(x) for x in spec.split(":"))
+    for seed in range(lo, hi):
+        print(f"sweep seed {seed}", flush=True)
+        test_fused_random_shapes(oracle, seed)
+        test_paged_random_shapes(seed)
+        test_wide_random_shapes(oracle, seed)
+        test_paged_wide_random_shapes(seed)
+        test_fused_random_shapes_with_device_lengths(oracle, seed)
