@@ -126,6 +126,7 @@ def bench_lib():
     lib = C.CDLL(path)
     lib.hw_stream_read.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_void_p]
     lib.hw_stream_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    lib.hw_stream_read_shaped.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p, C.c_int, C.c_void_p]
     return lib
 
 
@@ -307,6 +308,15 @@ def profile_mode(args, dev, stream, step_fn, kv_bytes, name):
         for _ in range(3):
             _lib.check(blib.hw_stream_read(big.data_ptr(), big.numel(), sink.data_ptr(), s_handle), "hw_stream_read")
             _lib.check(blib.hw_stream_copy(big.data_ptr() + half, big.data_ptr(), half, s_handle), "hw_stream_copy")
+        torch.cuda.synchronize()
+        # the control of the counter passes: a bare read of the workload's own byte count in the attention kernel's launch
+        # shape (one 256-thread workgroup per compute unit), walking the 512 MiB buffer
+        kvb16 = kv_bytes // 16 * 16
+        nbare = max(1, big.numel() // kvb16)
+        cus = _lib.lib.hw_device_cus()
+        for i in range(args.profile_steps):
+            _lib.check(blib.hw_stream_read_shaped(big.data_ptr() + (i % nbare) * kvb16, kvb16, sink.data_ptr(), cus, s_handle),
+                       "hw_stream_read_shaped")
         torch.cuda.synchronize()
     print(json.dumps({"profile_mode": True, "workload": name, "steps": args.profile_steps, "kv_bytes_per_step": kv_bytes,
                       "calibration": {"stream_read_bytes": 2 * half, "stream_copy_bytes_each_way": half}}))

@@ -16,6 +16,9 @@ extern "C" {
 /* Streaming read of `bytes` bytes (multiple of 16) from `src`, xor-reduced into sink[0..255]: the plain
    bandwidth calibration the attention kernel is compared with. */
 int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream);
+/* The same read with a given number of 256-thread workgroups (hw_stream_read launches 2048): the control for counter
+   passes on a kernel that runs one workgroup per compute unit. */
+int hw_stream_read_shaped(const void* src, size_t bytes, uint32_t* sink, int workgroups, void* stream);
 /* Plain copy kernel of known size, used to scale the FETCH_SIZE / WRITE_SIZE hardware counters. */
 int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream);
 

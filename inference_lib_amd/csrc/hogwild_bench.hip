@@ -40,6 +40,15 @@ int hw_stream_read(const void* src, size_t bytes, uint32_t* sink, void* stream) 
     return (int)hipGetLastError();
 }
 
+int hw_stream_read_shaped(const void* src, size_t bytes, uint32_t* sink, int workgroups, void* stream) {
+    if (src == nullptr || sink == nullptr) return HW_ERR_NULL;
+    if (bytes % 16 != 0 || !aligned16(src)) return HW_ERR_ALIGN;
+    if (workgroups < 1 || workgroups > 65536) return HW_ERR_SHAPE;
+    hipLaunchKernelGGL(stream_read_kernel, dim3(workgroups), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       reinterpret_cast<const u32x4*>(src), bytes / 16, sink);
+    return (int)hipGetLastError();
+}
+
 int hw_stream_copy(void* dst, const void* src, size_t bytes, void* stream) {
     if (src == nullptr || dst == nullptr) return HW_ERR_NULL;
     if (bytes % 16 != 0 || !aligned16(src) || !aligned16(dst)) return HW_ERR_ALIGN;

@@ -84,6 +84,11 @@ constexpr float NEG_BIG = -1.0e30f;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Workgroup barrier for data exchanged through LDS only: waits for this wave's LDS operations, not for its outstanding
+// global loads and global->LDS transfers.  (__syncthreads() carries a release fence, and the compiler makes every
+// transfer into LDS issued before it land first: a K/V tile in flight would be drained at every barrier.)
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Reductions over the four lanes {l, l^16, l^32, l^48}: the four quarter-waves hold different tokens of one row.
 // v_permlane32_swap / v_permlane16_swap exchange half-waves / 16-lane rows between two registers; applied to two
 // copies of a value they leave "mine" in one register and "my partner's" in the other, in every lane, without the
@@ -120,6 +125,24 @@ __device__ __forceinline__ float quarter_sum(float v) {
     v = a + b;
     quarter_pairs(v, 16, a, b);
     return a + b;
+}
+
+// Maximum / minimum over the 16 lanes of a row (lane % 16 = query row; the four rows of a wave hold the same values) by
+// four data-parallel-primitive moves: the two lane swaps within a quad, then the mirrored half row and the mirrored row.
+// (A generic shuffle goes through the LDS crossbar: four dependent round trips instead.)
+template <int CTRL>
+__device__ __forceinline__ int row_dpp(int v) { return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false); }
+__device__ __forceinline__ int row_max16(int v) {
+    v = max(v, row_dpp<0xB1>(v));     // quad_perm [1,0,3,2]
+    v = max(v, row_dpp<0x4E>(v));     // quad_perm [2,3,0,1]
+    v = max(v, row_dpp<0x141>(v));    // row_half_mirror
+    return max(v, row_dpp<0x140>(v)); // row_mirror
+}
+__device__ __forceinline__ int row_min16(int v) {
+    v = min(v, row_dpp<0xB1>(v));
+    v = min(v, row_dpp<0x4E>(v));
+    v = min(v, row_dpp<0x141>(v));
+    return min(v, row_dpp<0x140>(v));
 }
 
 // token (relative to the tile start) held in reduction slot `idx` (0..7) of quarter-wave `q`:
@@ -805,7 +828,7 @@ struct QueryRotation {
             const bool pad = r0 + rr >= a.R;   // padding rows of the 16-row MFMA block hold zeros
             const u32x4 z = {0, 0, 0, 0};
             if constexpr (PRE) {
-                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : xa[it];
+                if (q_lds != nullptr) *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : xa[it];
             } else {
                 float x1[CH], x2[CH], y1[CH], y2[CH];
                 Chunk<DT>::unpack(xa[it], x1);
@@ -817,13 +840,98 @@ struct QueryRotation {
                     y2[i] = x2[i] * c + x1[i] * sv;
                 }
                 const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
-                *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : ya;
-                *reinterpret_cast<u32x4*>(lrow + (slot + IPR) * 16) = pad ? z : yb;
+                if (q_lds != nullptr) {     // (null: the rotated queries are only wanted in memory)
+                    *reinterpret_cast<u32x4*>(lrow + slot * 16) = pad ? z : ya;
+                    *reinterpret_cast<u32x4*>(lrow + (slot + IPR) * 16) = pad ? z : yb;
+                }
                 if (write_rq && !pad) {
                     const RowMap rm = map_row(a, r0 + rr, hkv, GQ);
                     HW_GLOBAL char* rqp = a.rq + (f * fstride + rm.qrow * E) * SZ;
                     *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + slot * 16) = ya;
                     *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (slot + IPR) * 16) = yb;
+                }
+            }
+        }
+    }
+};
+
+// The same rotation done by every wave for itself, in the registers that hold the result as MFMA B operand: lane
+// (n = lane % 16, q = lane / 16) holds, for each 16-row block rb, the 16-byte chunks 4j + q (j < KJ) of query row
+// rb * 16 + n, and a rotation pair (e, e + E/2) is the chunk pair (4j + q, 4(j + KJ/2) + q): both in the same lane.  So
+// a wave loads its own operands (and the cos/sin values of their first-half chunks, and its rows' locations) straight
+// from memory, rotates them when they have arrived and starts on its tiles: no staging through LDS, no barrier, no
+// waiting for the other waves of the workgroup.  The four waves load the same few KB (served by the L1).
+template <class DT, int E, int RB, bool PRE>
+struct LaneRotation {
+    static constexpr int SZ = Elem<DT>::size;
+    static constexpr int CH = Chunk<DT>::CH;
+    static constexpr int KJ = E * SZ / 64;
+    static constexpr int HJ = KJ / 2;
+    static_assert(KJ % 2 == 0, "a rotation pair lies in one lane");
+
+    u32x4 x[RB][KJ];
+    f32x4 cs[PRE ? 1 : RB][PRE ? 1 : HJ][CH / 4], sn[PRE ? 1 : RB][PRE ? 1 : HJ][CH / 4];
+    int lc[RB];
+
+    __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int n, int q) {
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            // rows beyond R (MFMA padding) read the first row: harmless, and keeps the loads unconditional
+            const int row = r0 + rb * 16 + n;
+            const RowMap rm = map_row(a, row < a.R ? row : r0, hkv, GQ);
+            const HW_GLOBAL char* qp = a.q + (rm.qrow * E + (PRE ? f * fstride : 0)) * SZ;
+#pragma unroll
+            for (int j = 0; j < KJ; ++j) x[rb][j] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (4 * j + q) * 16);
+            if constexpr (!PRE) {
+#pragma unroll
+                for (int j = 0; j < HJ; ++j) {
+                    const size_t co = ((size_t)f * a.W * a.S + rm.ws) * E + (4 * j + q) * CH;
+#pragma unroll
+                    for (int i = 0; i < CH / 4; ++i) {
+                        cs[rb][j][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.cos + co + 4 * i);
+                        sn[rb][j][i] = *reinterpret_cast<const HW_GLOBAL f32x4*>(a.sin + co + 4 * i);
+                    }
+                }
+            }
+            lc[rb] = a.loc[(size_t)f * a.W * a.S + rm.ws];
+        }
+    }
+
+    // qreg[rb * KJ + j] = the operand of k-step j; lim[rb] = the row's visible length in this fragment of L tokens
+    __device__ __forceinline__ void finish(const DevHeader& a, u32x4* qreg, int (&lim)[RB], int f, int hkv, int r0, int GQ, int L,
+                                           bool write_rq, int n, int q) const {
+        const size_t fstride = (size_t)a.W * a.Hq * a.S * E;
+        const u32x4 z = {0, 0, 0, 0};
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            const int row = r0 + rb * 16 + n;
+            const bool pad = row >= a.R;          // padding rows of the 16-row MFMA block hold zeros and "see everything"
+            lim[rb] = pad ? 0x7fffffff : min(L, max(0, lc[rb] + 1));
+            if constexpr (PRE) {
+#pragma unroll
+                for (int j = 0; j < KJ; ++j) qreg[rb * KJ + j] = pad ? z : x[rb][j];
+            } else {
+                HW_GLOBAL char* rqp = nullptr;
+                if (write_rq && !pad) rqp = a.rq + (f * fstride + map_row(a, row, hkv, GQ).qrow * E) * SZ;
+#pragma unroll
+                for (int j = 0; j < HJ; ++j) {
+                    float x1[CH], x2[CH], y1[CH], y2[CH];
+                    Chunk<DT>::unpack(x[rb][j], x1);
+                    Chunk<DT>::unpack(x[rb][j + HJ], x2);
+#pragma unroll
+                    for (int i = 0; i < CH; ++i) {
+                        const float c = cs[rb][j][i >> 2][i & 3], sv = sn[rb][j][i >> 2][i & 3];
+                        y1[i] = x1[i] * c - x2[i] * sv;
+                        y2[i] = x2[i] * c + x1[i] * sv;
+                    }
+                    const u32x4 ya = Chunk<DT>::pack(y1), yb = Chunk<DT>::pack(y2);
+                    qreg[rb * KJ + j] = pad ? z : ya;
+                    qreg[rb * KJ + j + HJ] = pad ? z : yb;
+                    if (rqp != nullptr) {
+                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (4 * j + q) * 16) = ya;
+                        *reinterpret_cast<HW_GLOBAL u32x4*>(rqp + (4 * (j + HJ) + q) * 16) = yb;
+                    }
                 }
             }
         }

@@ -42,11 +42,11 @@ namespace hw {
 
 // Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
 #ifdef HW_CLOCKS
-__device__ unsigned long long hw_clock_buf[4096 * 8];
+__device__ unsigned long long hw_clock_buf[4096 * 16];
 #define HW_MARK(i)                                                                                  \
     do {                                                                                            \
         if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
-            hw_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + (i)] = wall_clock64();         \
+            hw_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (i)] = wall_clock64();         \
     } while (0)
 #else
 #define HW_MARK(i) do { } while (0)
@@ -71,13 +71,19 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 
     typedef hw::Exchange<ROWS, EV> Ex;
     constexpr int SBYTES = NWAVES * G::KSTAGE;
-    __shared__ __attribute__((aligned(16))) char q_lds[ROWS * G::QSTR];
-    __shared__ int lim_lds[ROWS];
+    // With one wave per SIMD there are registers to spare: the query operands of a segment stay in them (QREG).  The fp32
+    // kernel with one row block goes further (LANEROT): every wave loads and rotates its own operands in those registers,
+    // no copy of the rotated rows in LDS and no barrier in the prologue of a segment (config 1: 7.35 -> 7.1 us).  With
+    // two row blocks of 16-bit queries the 26 loads per wave this takes, against 7, cost more than the barriers did.
+    constexpr bool QREG = MINW == 1;
+    constexpr bool LANEROT = QREG && !VS && G::SZ == 4 && RB == 1;
+    __shared__ __attribute__((aligned(16))) char q_lds[LANEROT ? 16 : ROWS * G::QSTR];
+    __shared__ int lim_lds[LANEROT ? 1 : ROWS];
     // One K staging slot per tile in flight, each a separate LDS object so that the wait for a slot's incoming
     // transfers does not extend to the other slots.  Kernels that run one workgroup per CU have LDS to spare and give
     // the epilogue exchange memory of its own, so that a wave can hand over its accumulators the moment it is done; in
     // the others the exchange reuses the memory of slot 0.
-    constexpr bool EXSEP = MINW == 1 && sizeof(Ex) + PF * SBYTES + ROWS * G::QSTR + 1024 <= 160 * 1024;
+    constexpr bool EXSEP = MINW == 1 && sizeof(Ex) + PF * SBYTES + (LANEROT ? 0 : ROWS * G::QSTR) + 1024 <= 160 * 1024;
     union Slot0 {
         char k[SBYTES];
         char ex[EXSEP ? 16 : sizeof(Ex)];
@@ -90,6 +96,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     static_assert(PF <= 3, "three staging slots");
 
     const int tid = threadIdx.x;
+    HW_MARK(8);
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
@@ -165,8 +172,10 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     int f = 0, L = 0, lt0 = 0, lt1 = 0;
     bool opens_fragment = false;       // this workgroup owns the fragment's first tile (and writes its rotated queries)
     FragView fv;
-    QueryRotation<DT, E, ROWS, G::QSTR, PRE> qrot;
+    QueryRotation<DT, E, LANEROT ? 1 : ROWS, G::QSTR, PRE> qrot;
+    LaneRotation<DT, E, LANEROT ? RB : 1, PRE> lrot;
     int lm = 0;
+    [[maybe_unused]] int hw_seg = 0;   // 0 while the first segment is open (selects the timestamp slots of the tuning build)
     TileRegs<DT, E, EV> tr[PF];
     auto open_segment = [&]() {
         f = __builtin_ctzll(todo);
@@ -186,11 +195,15 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
         opens_fragment = s0 == fb;
         // global loads in issue order: query/cos/sin/loc of this fragment first (few), then the first K/V tile; the
         // rotation then waits only for the former while the tile stays in flight
-        HW_MARK(6);
-        qrot.load(a, f, hkv, r0, GQ, tid);
-        HW_MARK(7);
-        // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
-        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
+        HW_MARK(hw_seg ? 9 : 6);
+        if constexpr (LANEROT) {
+            lrot.load(a, f, hkv, r0, GQ, n, q);
+        } else {
+            qrot.load(a, f, hkv, r0, GQ, tid);
+            // (every thread loads, with a clamped row: a load inside a divergent branch would be waited for on the spot)
+            lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + (tid & (ROWS - 1)), a.R - 1), a.magic_gq)];
+        }
+        HW_MARK(hw_seg ? 10 : 7);
         // the first tile is requested before the prologue, further look-ahead tiles after it: a wave stalls
         // while the memory pipeline accepts its requests, and the prologue should not sit behind that stall
         if (PF > 1) load_tile<DT, E, EV>(tr[0], fv, kslots[0], koff, lt0 * TILE, n, q, lt0 < lt1);
@@ -199,42 +212,40 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     if (more) open_segment();
 
     while (more) {
-        HW_MARK(1);
-        // ---- prologue: rotate the queries of this fragment into LDS ----
-        __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
-        qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
-        // rows that pad the MFMA block get "sees everything": their query is zero and they are never stored,
-        // and they must not keep the unmasked fast path from being taken
-        if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
-        __syncthreads();
-
-        // with one wave per SIMD there are registers to spare: keep the query operands of the segment in them
-        constexpr bool QREG = MINW == 1;
+        HW_MARK(hw_seg ? 11 : 1);
+        // ---- prologue: rotate the queries of this fragment ----
         u32x4 qreg[QREG ? RB * G::KJ : 1];
-        if constexpr (QREG) {
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb)
-#pragma unroll
-                for (int j = 0; j < G::KJ; ++j)
-                    qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
-        }
         int lim[RB];
         int maxlim = 0, minlim = 0x7fffffff;
+        if constexpr (LANEROT) {
+            lrot.finish(a, qreg, lim, f, hkv, r0, GQ, L, a.rq != nullptr && opens_fragment && wv == 0, n, q);
+        } else {
+            // (barriers for LDS only: __syncthreads() would make the K transfers of the tile in flight land first)
+            lds_barrier();     // previous segment's readers are done with q_lds / lim_lds
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
+            // rows that pad the MFMA block get "sees everything": their query is zero and they are never stored,
+            // and they must not keep the unmasked fast path from being taken
+            if (tid < ROWS) lim_lds[tid] = (r0 + tid < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
+            lds_barrier();
+            if constexpr (QREG) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+                    for (int j = 0; j < G::KJ; ++j)
+                        qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+            }
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) lim[rb] = lim_lds[rb * 16 + n];
+        }
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-            lim[rb] = lim_lds[rb * 16 + n];
             const bool pad = r0 + rb * 16 + n >= a.R;
             maxlim = max(maxlim, pad ? 0 : lim[rb]);
             minlim = min(minlim, lim[rb]);
         }
-#pragma unroll
-        for (int off = 1; off < 16; off <<= 1) {
-            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
-            minlim = min(minlim, __shfl_xor(minlim, off, 64));
-        }
-        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
-        minlim = __builtin_amdgcn_readfirstlane(minlim);
-        HW_MARK(2);
+        maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
+        minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
+        HW_MARK(hw_seg ? 12 : 2);
 #pragma unroll
         for (int i = 1; i < PF - 1; ++i)
             load_tile<DT, E, EV>(tr[i], fv, kslots[i], koff, (lt0 + i * NWAVES) * TILE, n, q, lt0 + i * NWAVES < lt1);
@@ -272,6 +283,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
             }
         }
         more = todo != 0;
+        HW_MARK(hw_seg ? 14 : 13);
+        hw_seg = 1;
         if (more) open_segment();
     }
 
@@ -290,7 +303,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
             __syncthreads();
             QueryRotation<DT, E, ROWS, G::QSTR, PRE> qempty;
             qempty.load(a, f, hkv, r0, GQ, tid);
-            qempty.finish(a, q_lds, f, hkv, r0, GQ, true, tid);
+            qempty.finish(a, LANEROT ? nullptr : q_lds, f, hkv, r0, GQ, true, tid);
         }
     }
 }

@@ -31,7 +31,7 @@ def test_calibration_kernels_live_in_their_own_library():
     L = _lib()
     header = open(os.path.join(ROOT, "include", "hogwild_bench.h")).read()
     declared = set(re.findall(r"^\s*int\s+(hw_\w+)\s*\(", header, flags=re.M))
-    assert declared == {"hw_stream_read", "hw_stream_copy"}, declared
+    assert declared == {"hw_stream_read", "hw_stream_read_shaped", "hw_stream_copy"}, declared
     bench = C.CDLL(os.path.join(ROOT, "inference_lib_amd", "libhogwild_bench.so"))
     for name in declared:
         assert hasattr(bench, name), name
