@@ -109,7 +109,14 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     ka.h.wgs_per_head = plan.wgs_per_head;
     ka.h.nwg = plan.workgroups;
     ka.h.prerotated = prerotated ? 1 : 0;
-    ka.h.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
+    // One workgroup per kv head and row group holds whole rows: it writes out / lse itself and the merge launch is
+    // dropped (the 128-row kernel has an epilogue of its own and always goes through the merge).
+    const bool direct = plan.wgs_per_head == 1 && stages == (HW_STAGE_ATTENTION | HW_STAGE_MERGE) && plan.row_blocks != hw::WIDE_ROW_BLOCKS;
+    ka.h.flags = ((plan.workgroups % 8 == 0) ? hw::KH_XCD_REMAP : 0) | (direct ? hw::KH_DIRECT : 0);
+    if (direct) {
+        ka.h.part_o = reinterpret_cast<float*>(p->out);
+        ka.h.part_ml = p->lse;
+    }
     ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
     // multipliers for the in-kernel divisions (exact for numerators < 2^20 and divisors < 2^12, both validated)
     auto magic = [](int d) { return magic_of(d); };
@@ -126,7 +133,7 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
             e = hw::launch_attention(ka, p->dtype, p->E, plan.row_blocks, p->variant, stream);
         if (e != hipSuccess) return (int)e;
     }
-    if (!(stages & HW_STAGE_MERGE)) return (int)e;
+    if (!(stages & HW_STAGE_MERGE) || direct) return (int)e;
     hw::MergeArgs ma;
     ma.part_o = ka.h.part_o;
     ma.part_ml = ka.h.part_ml;

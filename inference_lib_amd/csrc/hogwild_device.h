@@ -564,9 +564,14 @@ struct Exchange {
 // ALIASED: `ex` shares its memory with a K staging slot, so nobody may write it before every wave is done with its
 // tiles; otherwise each wave hands over as soon as it is done, while the slower waves of the workgroup still compute.
 // Rows beyond `nrows` (MFMA padding) are neither written nor read.
+// `direct` (uniform over the launch): the workgroup holds everything its rows will ever see (one workgroup per kv head and
+// row group), so the combined rows are normalised here and written as the operator's result: part_o is then the
+// address of out, part_ml that of lse (or null), and orow[rb] the lane's output row (row index of out / lse) in row
+// block rb.  The arithmetic is that of the merge kernel on a single partial, bit for bit.
 template <class DT, int EV, int RB, bool ALIASED>
 __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Exchange<RB * 16, EV>& ex, int wv, int n, int q, int tid,
-                                               HW_GLOBAL float* part_o, HW_GLOBAL float* part_ml, size_t part, int nrows) {
+                                               HW_GLOBAL float* part_o, HW_GLOBAL float* part_ml, size_t part, int nrows,
+                                               bool direct = false, const size_t* orow = nullptr) {
     constexpr int NOC = EV / 16;
     constexpr int NSLOT = RB * NOC;
     constexpr int SPW = NSLOT / NWAVES;       // accumulators each wave combines
@@ -608,7 +613,14 @@ __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Excha
         float wgt[NWAVES];
 #pragma unroll
         for (int w2 = 0; w2 < NWAVES; ++w2) wgt[w2] = fast_exp2(m4[w2] - mm);
+        float lsum = 0.f;
+#pragma unroll
+        for (int w2 = 0; w2 < NWAVES; ++w2) lsum = __builtin_fmaf(l4[w2], wgt[w2], lsum);
+        typedef typename Elem<DT>::store_t store_t;
+        const size_t orw = direct ? orow[rb] : 0;
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
         HW_GLOBAL float* dst = part_o + (part + row) * EV;
+        HW_GLOBAL store_t* odst = reinterpret_cast<HW_GLOBAL store_t*>(part_o) + orw * EV;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float run[SPW];
@@ -619,16 +631,20 @@ __device__ __forceinline__ void store_partials(WaveState<RB, EV / 16>& st, Excha
                 for (int w2 = 1; w2 < NWAVES; ++w2) acc = __builtin_fmaf(ov[j][w2][i], wgt[w2], acc);
                 run[j] = acc;
             }
-            HW_GLOBAL float* d = dst + out_ev<DT, EV>(c0, 4 * q + i);    // chunks c0 .. c0+SPW-1 are consecutive floats from here
-            if constexpr (SPW == 4) *reinterpret_cast<HW_GLOBAL f32x4*>(d) = f32x4{run[0], run[1], run[2], run[3]};
-            else if constexpr (SPW == 2) *reinterpret_cast<HW_GLOBAL f32x2*>(d) = f32x2{run[0], run[1]};
-            else *d = run[0];
+            const int e0 = out_ev<DT, EV>(c0, 4 * q + i);    // chunks c0 .. c0+SPW-1 are consecutive elements from here
+            if (direct) {
+#pragma unroll
+                for (int j = 0; j < SPW; ++j) odst[e0 + j] = Elem<DT>::from_float(run[j] * inv);
+            } else {
+                HW_GLOBAL float* d = dst + e0;
+                if constexpr (SPW == 4) *reinterpret_cast<HW_GLOBAL f32x4*>(d) = f32x4{run[0], run[1], run[2], run[3]};
+                else if constexpr (SPW == 2) *reinterpret_cast<HW_GLOBAL f32x2*>(d) = f32x2{run[0], run[1]};
+                else *d = run[0];
+            }
         }
         if (q == 0 && c0 == 0) {
-            float lsum = 0.f;
-#pragma unroll
-            for (int w2 = 0; w2 < NWAVES; ++w2) lsum = __builtin_fmaf(l4[w2], wgt[w2], lsum);
-            *reinterpret_cast<HW_GLOBAL f32x2*>(part_ml + (part + row) * 2) = f32x2{mm, lsum};
+            if (!direct) *reinterpret_cast<HW_GLOBAL f32x2*>(part_ml + (part + row) * 2) = f32x2{mm, lsum};
+            else if (part_ml != nullptr) part_ml[orw] = lsum > 0.f ? (mm + __builtin_amdgcn_logf(lsum)) * 0.69314718055994530942f : -__builtin_inff();
         }
     }
 }
@@ -648,7 +664,7 @@ struct DevHeader {
     int F, W, Hq, Hkv, S, R;
     int nrg, wgs_per_head, nwg;
     int prerotated;
-    int xcd_remap;
+    int flags;
     float sc;
     unsigned magic_gq, magic_s, magic_nrg, magic_wg;
 };

@@ -36,11 +36,14 @@ struct alignas(64) KernelHeader {
     int F, W, Hq, Hkv, S, R;
     int nrg, wgs_per_head, nwg;
     int prerotated;
-    int xcd_remap;
+    int flags;          // KH_XCD_REMAP | KH_DIRECT
     float sc;           // scale * log2(e)
     unsigned magic_gq, magic_s, magic_nrg, magic_wg;   // ceil(2^32 / d) for d = Hq/Hkv, S, nrg, wgs_per_head
 };
 static_assert(sizeof(KernelHeader) == 128, "KernelHeader must be 32 dwords");
+constexpr int KH_XCD_REMAP = 1;   // consecutive logical workgroup ids share an XCD (the grid is a multiple of 8)
+constexpr int KH_DIRECT = 2;      // one workgroup per kv head and row group: it normalises its own result and writes out / lse
+                                  // itself (part_o then holds the address of out, part_ml that of lse or null); no merge launch
 
 struct KernelArgs {
     KernelHeader h;

@@ -145,7 +145,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 
     // consecutive logical ids stay on one XCD (hardware deals workgroups round-robin over the 8 XCDs)
     int bid = blockIdx.x;
-    if (a.xcd_remap) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
+    if (a.flags & KH_XCD_REMAP) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
     const int hg = fast_div(bid, a.magic_nrg);            // (kv head, split) pair
     const int rg = bid - hg * a.nrg;
     const int hkv = fast_div(hg, a.magic_wg);
@@ -290,8 +290,12 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
 
     HW_MARK(3);
     // ---- merge the four waves of the workgroup and store the partial of this workgroup ----
+    const bool direct = (a.flags & KH_DIRECT) != 0;
+    size_t orow[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) orow[rb] = direct ? map_row(a, min(r0 + rb * 16 + n, a.R - 1), hkv, GQ).qrow : 0;
     store_partials<DT, EV, RB, !EXSEP>(st, ex, wv, n, q, tid, a.part_o, a.part_ml, (size_t)(hkv * a.wgs_per_head + g) * a.R + r0,
-                               min(ROWS, a.R - r0));
+                               min(ROWS, a.R - r0), direct, orow);
     HW_MARK(5);
 
     // rotated queries of zero-length fragments are still part of the operator's visible output

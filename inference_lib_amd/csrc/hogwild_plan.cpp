@@ -103,6 +103,14 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
         // narrow kernels deal a workgroup's tiles to its four waves; in the wide kernel every wave takes every tile
         const int by_work = wide ? (int)((tiles + 3) / 4) : (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
         if (wgs > by_work) wgs = by_work;
+        // Small problems in 16-bit types: one workgroup per kv head (and row group) holds whole rows, writes the result
+        // itself and saves the merge launch (~2.4 us), which is worth more than what the split buys as long as its
+        // fragments, opened one after the other, stay few: measured, single fragments of up to 16 tiles 5.8-7.0 us
+        // against 8.0-8.2 us, three fragments of 6 / 8 tiles 8.4 / 8.7 against 8.9, of 15 tiles 9.4 against 7.4.  (The
+        // fp32 kernel takes ~1 us per tile and loses beyond the 4 tiles that give one workgroup anyway.)
+        int nonempty = 0;
+        for (int f = 0; f < p->F; ++f) nonempty += p->len[f] > 0 ? 1 : 0;
+        if (!wide && p->dtype != HW_F32 && tiles + 6ll * (nonempty > 0 ? nonempty - 1 : 0) <= 20) wgs = 1;
     }
     if (wgs > (int)tiles) wgs = (int)tiles;
     if (wgs > hw::MAX_SPLITS) wgs = hw::MAX_SPLITS;

@@ -232,7 +232,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
 
     int bid = blockIdx.x;
-    if (a.xcd_remap) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
+    if (a.flags & KH_XCD_REMAP) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
     const int hg = fast_div(bid, a.magic_nrg);
     const int rg = bid - hg * a.nrg;
     const int hkv = fast_div(hg, a.magic_wg);
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     a.len_dev = nullptr;
     a.F = ph.F; a.W = ph.LW; a.Hq = ph.Hq; a.Hkv = ph.Hkv; a.S = ph.LS; a.R = rend;
     a.nrg = 1; a.wgs_per_head = ph.nsplit; a.nwg = ph.nwg;
-    a.prerotated = 1; a.xcd_remap = 0; a.sc = ph.sc;
+    a.prerotated = 1; a.flags = 0; a.sc = ph.sc;
     a.magic_gq = ph.magic_gq; a.magic_s = ph.magic_ls; a.magic_nrg = 0; a.magic_wg = 0;
 
     // The sequence's block table goes into LDS once: per tile every lane then looks up the block of its own position

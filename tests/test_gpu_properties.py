@@ -186,6 +186,45 @@ def test_two_stages_equal_the_fused_call():
     assert torch.equal(out1, out2) and torch.equal(lse1, lse2)
 
 
+@pytest.mark.parametrize("dtype,W,S,Hq,Hkv,E,lens", [
+    ("bf16", 2, 1, 8, 2, 128, (128, 0, 0)),            # 4 tiles: one workgroup per head by itself
+    ("f16", 2, 1, 8, 2, 64, (500, 0, 0)),              # 16 tiles in one fragment: the planner prefers one workgroup
+    ("bf16", 3, 2, 12, 4, 128, (100, 0, 33, 57)),      # three short fragments, an empty one, 18 rows
+    ("f32", 2, 1, 8, 2, 64, (64, 20, 5)),              # fp32, 4 tiles
+    ("f16", 4, 3, 8, 2, 128, (64, 30, 0, 0, 31)),      # 48 rows per kv head: two row groups, each writing its rows
+])
+def test_one_workgroup_per_head_writes_the_result_itself(oracle, dtype, W, S, Hq, Hkv, E, lens):
+    """A plan with one workgroup per kv head normalises in the attention kernel and launches no merge; the result is
+    that of the two stages (attention kernel into the workspace, merge kernel) bit for bit, and the oracle's within the
+    usual tolerance."""
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype=dtype, W=W, S=S, Hq=Hq, Hkv=Hkv, E=E, lens=lens, seed=41)
+    pl = _lib.plan(list(lens), W=W, S=S, Hq=Hq, Hkv=Hkv, Ev=E, num_cus=256,
+                   dtype={"f32": _lib.HW_F32, "f16": _lib.HW_F16, "bf16": _lib.HW_BF16}[dtype])
+    assert pl.wgs_per_head == 1
+    cd = c.to(_dev())
+    out1 = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    out2 = torch.full_like(out1, float("nan"))
+    lse1 = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    lse2 = torch.full_like(lse1, float("nan"))
+    p1 = _problem(cd, out1, lse=lse1)
+    ws = torch.full((p1.workspace_bytes(),), 0xAB, dtype=torch.uint8, device=_dev())
+    p1.set_workspace(ws)
+    p1.run()
+    torch.cuda.synchronize()
+    assert bool((ws == 0xAB).all())                      # the single launch leaves the workspace alone
+    p2 = _problem(cd, out2, lse=lse2)
+    p2.run(stages=1)
+    torch.cuda.synchronize()
+    assert torch.isnan(out2.float()).all()
+    p2.run(stages=2)
+    torch.cuda.synchronize()
+    assert torch.equal(out1.view(torch.uint8), out2.view(torch.uint8)) and torch.equal(lse1.view(torch.uint8), lse2.view(torch.uint8))
+    want_o, want_l, _ = oracle_fused(oracle, c)
+    assert_close("out", out1, want_o, TOL[dtype])
+    assert_close("lse", lse1, want_l, TOL[dtype])
+
+
 def test_side_stream_and_concurrent_streams(oracle):
     from inference_lib_amd import cases
     ca = cases.small_case(dtype="bf16", W=2, S=1, Hq=8, Hkv=2, E=128, lens=(900, 300, 411), seed=31)
