@@ -40,9 +40,12 @@
 extern "C" {
 #endif
 
-#define HW_ABI_VERSION 4
-#define HW_MAX_FRAGMENTS 64
-#define HW_MAX_SPLITS 256      /* workgroups per kv head */
+#define HW_ABI_VERSION 5
+#define HW_MAX_FRAGMENTS 512          /* fragments per call, the reference's limit (src/binding.cu:79-82) */
+#define HW_MAX_LAUNCH_FRAGMENTS 64    /* fragments one attention launch takes (their table travels in the kernel arguments);
+                                         a call with more runs ceil(F / 64) attention launches, whose split-K partials lie
+                                         side by side in the workspace, and one merge over all of them */
+#define HW_MAX_SPLITS 256             /* workgroups per kv head and launch */
 
 typedef enum hw_status {
     HW_OK = 0,
@@ -51,7 +54,7 @@ typedef enum hw_status {
     HW_ERR_SHAPE = -3,         /* a dimension is non-positive or inconsistent (Hq % Hkv, RotE > E, odd RotE, a fragment
                                   whose kv-head slice reaches 2 GiB, scale not positive and finite, ...) */
     HW_ERR_UNSUPPORTED = -4,   /* shape is valid but no kernel is instantiated for it (never a silent no-op) */
-    HW_ERR_FRAGMENTS = -5,     /* F < 1 or F > HW_MAX_FRAGMENTS */
+    HW_ERR_FRAGMENTS = -5,     /* F < 1 or F > HW_MAX_FRAGMENTS (HW_MAX_LAUNCH_FRAGMENTS where stated) */
     HW_ERR_WORKSPACE = -6,     /* workspace NULL or smaller than hw_workspace_bytes() */
     HW_ERR_ALIGN = -7,         /* a device pointer is not 16-byte aligned */
     HW_ERR_NO_DEVICE = -8,     /* no usable HIP device */
@@ -79,8 +82,8 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   len_dev    optional DEVICE array of F current lengths (hw_fused_attention with RotE == E only).  With it, len[f] is
  *              the bound the split is planned for and the buffers must hold (cap[f] >= len[f]), and fragment f has
  *              min(len[f], len_dev[f]) tokens when the kernel runs: a launch captured in a HIP graph stays valid while
- *              the segments grow up to len[f].  No counterpart in the reference, whose segments are re-allocated by
- *              torch.cat on every update (python/hogwild/attention.py:148-158).
+ *              the segments grow up to len[f].  F <= HW_MAX_LAUNCH_FRAGMENTS.  No counterpart in the reference, whose
+ *              segments are re-allocated by torch.cat on every update (python/hogwild/attention.py:148-158).
  *   workspace  device scratch of at least hw_workspace_bytes() bytes, caller-owned, 16-byte aligned
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
@@ -126,7 +129,7 @@ typedef struct hw_plan {
     int32_t tiles_per_head;   /* sum_f ceil(len[f] / tile_tokens) */
     int32_t wgs_per_head;     /* split-K factor */
     int32_t workgroups;       /* grid size of the attention kernel */
-    int32_t tile_begin[HW_MAX_FRAGMENTS + 1];   /* first tile of each fragment in a head's tile sequence */
+    int32_t tile_begin[HW_MAX_LAUNCH_FRAGMENTS + 1];   /* first tile of each fragment in a head's tile sequence */
     int32_t wg_tile_begin[HW_MAX_SPLITS + 1];   /* first tile of each workgroup; balanced by tiles + a fixed
                                                     cost for every fragment a workgroup has to open */
     size_t workspace_bytes;
@@ -138,7 +141,8 @@ const char* hw_status_string(int status);
 /* Host-only argument check shared by all entry points (pointer checks cover what `fused` != 0 needs). */
 int hw_validate(const hw_problem* p, int fused);
 
-/* Host-only: the split plan for a device with `num_cus` compute units. */
+/* Host-only: the split plan of one attention launch for a device with `num_cus` compute units
+   (F <= HW_MAX_LAUNCH_FRAGMENTS; a call with more fragments plans each group of 64 like this). */
 int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan);
 
 /* Workspace size for the current device: what hw_fused_attention needs for this problem (if the rotary width is not
@@ -295,7 +299,7 @@ int hw_build_inputs_dev(int32_t* locations, float* cosines, float* sines, const 
                         const float* inv_freq, float attention_scaling, int round_dtype, int F, int W, int S, int RotE,
                         void* stream);
 
-/* len_dev[f] += add[f] for f < F <= HW_MAX_FRAGMENTS (add is a HOST array): the first node of a captured decode step. */
+/* len_dev[f] += add[f] for f < F <= HW_MAX_LAUNCH_FRAGMENTS (add is a HOST array): the first node of a captured decode step. */
 int hw_advance_lengths(int32_t* len_dev, const int32_t* add, int F, void* stream);
 
 #define HW_ROPE_EAGER 0   /* every product and the sum rounded as an eager tensor expression rounds them: bit-identical to

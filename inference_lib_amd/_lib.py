@@ -15,7 +15,9 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
 
-HW_MAX_FRAGMENTS = 64
+HW_MAX_FRAGMENTS = 512          # per call
+HW_MAX_LAUNCH_FRAGMENTS = 64    # per attention launch (what hw_plan describes)
+HW_ABI_VERSION = 5              # the version the structures below mirror
 HW_MAX_SPLITS = 256
 HW_STATIC_SCRATCH_BYTES = 8 << 20
 HW_F32, HW_F16, HW_BF16 = 0, 1, 2
@@ -51,7 +53,7 @@ class HwPlan(C.Structure):
     _fields_ = [
         ("rows", C.c_int32), ("row_blocks", C.c_int32), ("row_groups", C.c_int32), ("tile_tokens", C.c_int32),
         ("tiles_per_head", C.c_int32), ("wgs_per_head", C.c_int32), ("workgroups", C.c_int32),
-        ("tile_begin", C.c_int32 * (HW_MAX_FRAGMENTS + 1)),
+        ("tile_begin", C.c_int32 * (HW_MAX_LAUNCH_FRAGMENTS + 1)),
         ("wg_tile_begin", C.c_int32 * (HW_MAX_SPLITS + 1)),
         ("workspace_bytes", C.c_size_t),
     ]
@@ -124,6 +126,9 @@ def _load() -> C.CDLL:
             "(there is no fallback path for the Hogwild attention operators)")
     lib = C.CDLL(LIB_PATH)
     lib.hw_version.restype = C.c_int
+    if lib.hw_version() != HW_ABI_VERSION:      # a stale library would be driven with structures of another layout
+        raise ImportError(f"{LIB_PATH} has ABI version {lib.hw_version()}, this module mirrors version {HW_ABI_VERSION}: "
+                          "rebuild it with `python -m inference_lib_amd.build`")
     lib.hw_status_string.restype = C.c_char_p
     lib.hw_status_string.argtypes = [C.c_int]
     lib.hw_validate.argtypes = [C.POINTER(HwProblem), C.c_int]

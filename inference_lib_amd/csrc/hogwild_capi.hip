@@ -63,70 +63,79 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     int cus = 0;
     st = device_cus(&cus);
     if (st != HW_OK) return st;
-    hw_plan plan;
-    st = make_plan(p, cus, &plan, fused);
+    CallPlan cp;
+    st = plan_call(p, cus, &cp, fused);
     if (st != HW_OK) return st;
-    if (p->workspace == nullptr || p->workspace_bytes < plan.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
+    if (p->workspace == nullptr || p->workspace_bytes < cp.workspace_bytes || !aligned16(p->workspace)) return HW_ERR_WORKSPACE;
+    const hw_plan& plan0 = cp.plan[0];
     // the VALU logits exist for what they are measured on: the fused entry with full rotary width, one row block, host lengths
-    if (p->variant == HW_VARIANT_VALU_QK && (!fused || p->RotE != p->E || plan.row_blocks != 1 || p->len_dev != nullptr)) return HW_ERR_UNSUPPORTED;
+    if (p->variant == HW_VARIANT_VALU_QK && (!fused || p->RotE != p->E || plan0.row_blocks != 1 || p->len_dev != nullptr)) return HW_ERR_UNSUPPORTED;
 
     hipStream_t stream = reinterpret_cast<hipStream_t>(stream_);
-    const void* q_in = p->q;
+    const size_t esz = elem_size(p->dtype);
+    const char* q_in = reinterpret_cast<const char*>(p->q);
     bool prerotated = !fused;
     if (fused && p->RotE != p->E) {
         void* rqbuf = p->rq;
-        if (rqbuf == nullptr) {
-            const size_t rqbytes = ((size_t)p->F * p->W * p->Hq * p->S * p->E * elem_size(p->dtype) + 255) & ~(size_t)255;
-            rqbuf = reinterpret_cast<char*>(p->workspace) + (plan.workspace_bytes - rqbytes);
+        if (rqbuf == nullptr) rqbuf = reinterpret_cast<char*>(p->workspace) + cp.partial_bytes;
+        if (stages & HW_STAGE_ATTENTION) {
+            hipError_t er = hw::launch_rope(rqbuf, p->q, p->cosines, p->sines, p->dtype, p->F, p->W, p->Hq, p->S, p->E, p->RotE, stream);
+            if (er != hipSuccess) return (int)er;
         }
-        hipError_t er = hw::launch_rope(rqbuf, p->q, p->cosines, p->sines, p->dtype, p->F, p->W, p->Hq, p->S, p->E, p->RotE, stream);
-        if (er != hipSuccess) return (int)er;
-        q_in = rqbuf;
+        q_in = reinterpret_cast<const char*>(rqbuf);
         prerotated = true;
     }
-    hw::KernelArgs ka;
-    std::memset(&ka, 0, sizeof(ka));
-    for (int f = 0; f < p->F; ++f) {
-        ka.frag.k[f] = p->k[f];
-        ka.frag.v[f] = p->v[f];
-        ka.frag.lc[f].len = p->len[f];
-        ka.frag.lc[f].cap = p->cap != nullptr ? p->cap[f] : p->len[f];
-    }
-    for (int f = 0; f <= HW_MAX_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
-    for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];
-    ka.h.q = q_in;
-    ka.h.loc = p->locations;
-    ka.h.cos = p->cosines;
-    ka.h.sin = p->sines;
-    ka.h.rq = (fused && !prerotated) ? p->rq : nullptr;
-    const size_t parts = (size_t)p->Hkv * plan.wgs_per_head;
-    ka.h.part_o = reinterpret_cast<float*>(p->workspace);
-    ka.h.part_ml = ka.h.part_o + parts * plan.rows * p->Ev;
-    ka.h.len_dev = p->len_dev;
-    ka.h.F = p->F; ka.h.W = p->W; ka.h.Hq = p->Hq; ka.h.Hkv = p->Hkv; ka.h.S = p->S;
-    ka.h.R = plan.rows;
-    ka.h.nrg = plan.row_groups;
-    ka.h.wgs_per_head = plan.wgs_per_head;
-    ka.h.nwg = plan.workgroups;
-    ka.h.prerotated = prerotated ? 1 : 0;
+    const int rows = plan0.rows;
+    float* const part_o = reinterpret_cast<float*>(p->workspace);
+    float* const part_ml = part_o + (size_t)p->Hkv * cp.slots * rows * p->Ev;
     // One workgroup per kv head and row group holds whole rows: it writes out / lse itself and the merge launch is
     // dropped (the 128-row kernel has an epilogue of its own and always goes through the merge).
-    const bool direct = plan.wgs_per_head == 1 && stages == (HW_STAGE_ATTENTION | HW_STAGE_MERGE) && plan.row_blocks != hw::WIDE_ROW_BLOCKS;
-    ka.h.flags = ((plan.workgroups % 8 == 0) ? hw::KH_XCD_REMAP : 0) | (direct ? hw::KH_DIRECT : 0);
-    if (direct) {
-        ka.h.part_o = reinterpret_cast<float*>(p->out);
-        ka.h.part_ml = p->lse;
-    }
-    ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
-    // multipliers for the in-kernel divisions (exact for numerators < 2^20 and divisors < 2^12, both validated)
+    const bool direct = cp.groups == 1 && plan0.wgs_per_head == 1 && stages == (HW_STAGE_ATTENTION | HW_STAGE_MERGE) &&
+                        plan0.row_blocks != hw::WIDE_ROW_BLOCKS;
     auto magic = [](int d) { return magic_of(d); };
-    ka.h.magic_gq = magic(p->Hq / p->Hkv);
-    ka.h.magic_s = magic(p->S);
-    ka.h.magic_nrg = magic(plan.row_groups);
-    ka.h.magic_wg = magic(plan.wgs_per_head);
 
     hipError_t e = hipSuccess;
-    if (stages & HW_STAGE_ATTENTION) {
+    for (int gi = 0; gi < cp.groups && (stages & HW_STAGE_ATTENTION); ++gi) {
+        const hw_plan& plan = cp.plan[gi];
+        const int f0 = cp.first[gi], nf = cp.count[gi];
+        const size_t ws_rows = (size_t)p->W * p->S;                    // (worker, token) pairs per fragment
+        const size_t q_frag = ws_rows * p->Hq * p->E * esz;            // bytes of one fragment's rotated queries
+        hw::KernelArgs ka;
+        std::memset(&ka, 0, sizeof(ka));
+        for (int f = 0; f < nf; ++f) {
+            ka.frag.k[f] = p->k[f0 + f];
+            ka.frag.v[f] = p->v[f0 + f];
+            ka.frag.lc[f].len = p->len[f0 + f];
+            ka.frag.lc[f].cap = p->cap != nullptr ? p->cap[f0 + f] : p->len[f0 + f];
+        }
+        for (int f = 0; f <= HW_MAX_LAUNCH_FRAGMENTS; ++f) ka.frag.tile_begin[f] = plan.tile_begin[f];
+        for (int i = 0; i <= HW_MAX_SPLITS; ++i) ka.wg_tile[i] = plan.wg_tile_begin[i];
+        // everything indexed by fragment starts at this group's first fragment
+        ka.h.q = prerotated ? q_in + (size_t)f0 * q_frag : q_in;
+        ka.h.loc = p->locations + (size_t)f0 * ws_rows;
+        ka.h.cos = p->cosines != nullptr ? p->cosines + (size_t)f0 * ws_rows * p->RotE : nullptr;
+        ka.h.sin = p->sines != nullptr ? p->sines + (size_t)f0 * ws_rows * p->RotE : nullptr;
+        ka.h.rq = (fused && !prerotated && p->rq != nullptr) ? reinterpret_cast<char*>(p->rq) + (size_t)f0 * q_frag : nullptr;
+        ka.h.part_o = part_o + (size_t)cp.slot_base[gi] * rows * p->Ev;
+        ka.h.part_ml = part_ml + (size_t)cp.slot_base[gi] * rows * 2;
+        ka.h.len_dev = p->len_dev;
+        ka.h.F = nf; ka.h.W = p->W; ka.h.Hq = p->Hq; ka.h.Hkv = p->Hkv; ka.h.S = p->S;
+        ka.h.R = rows;
+        ka.h.nrg = plan.row_groups;
+        ka.h.wgs_per_head = plan.wgs_per_head;
+        ka.h.nwg = plan.workgroups;
+        ka.h.slot_stride = cp.slots;
+        ka.h.flags = ((plan.workgroups % 8 == 0) ? hw::KH_XCD_REMAP : 0) | (direct ? hw::KH_DIRECT : 0) | (prerotated ? hw::KH_PREROTATED : 0);
+        if (direct) {
+            ka.h.part_o = reinterpret_cast<float*>(p->out);
+            ka.h.part_ml = p->lse;
+        }
+        ka.h.sc = (float)((double)p->scale * 1.4426950408889634074);
+        // multipliers for the in-kernel divisions (exact for numerators < 2^20 and divisors < 2^12, both validated)
+        ka.h.magic_gq = magic(p->Hq / p->Hkv);
+        ka.h.magic_s = magic(p->S);
+        ka.h.magic_nrg = magic(plan.row_groups);
+        ka.h.magic_wg = magic(plan.wgs_per_head);
         if (plan.row_blocks == hw::WIDE_ROW_BLOCKS)
             e = hw::launch_attention_wide(ka, p->dtype, p->E, stream);
         else
@@ -135,13 +144,13 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     }
     if (!(stages & HW_STAGE_MERGE) || direct) return (int)e;
     hw::MergeArgs ma;
-    ma.part_o = ka.h.part_o;
-    ma.part_ml = ka.h.part_ml;
+    ma.part_o = part_o;
+    ma.part_ml = part_ml;
     ma.out = p->out;
     ma.lse = p->lse;
-    ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = plan.rows;
-    ma.wgs_per_head = plan.wgs_per_head;
-    ma.xcd_local = (plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
+    ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = rows;
+    ma.wgs_per_head = cp.slots;
+    ma.xcd_local = (cp.groups == 1 && plan0.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
     e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
     return (int)e;
 }
@@ -264,7 +273,7 @@ int build_inputs_run(int32_t* locations, float* cosines, float* sines, const int
 
 int build_inputs_dev_run(int32_t* locations, float* cosines, float* sines, const int32_t* len_dev, const int32_t* orders,
                          const float* inv_freq, float scaling, int round_dtype, int F, int W, int S, int RotE, void* stream) {
-    if (F < 1 || F > HW_MAX_FRAGMENTS || W < 1 || S < 1 || RotE < 0 || (RotE & 1)) return HW_ERR_SHAPE;
+    if (F < 1 || F > HW_MAX_LAUNCH_FRAGMENTS || W < 1 || S < 1 || RotE < 0 || (RotE & 1)) return HW_ERR_SHAPE;
     if (round_dtype != HW_F32 && round_dtype != HW_F16 && round_dtype != HW_BF16) return HW_ERR_DTYPE;
     if (locations == nullptr || len_dev == nullptr || orders == nullptr) return HW_ERR_NULL;
     if (RotE > 0 && (cosines == nullptr || sines == nullptr || inv_freq == nullptr)) return HW_ERR_NULL;
@@ -292,7 +301,7 @@ int build_inputs_dev_run(int32_t* locations, float* cosines, float* sines, const
 
 int advance_lengths_run(int32_t* len_dev, const int32_t* add, int F, void* stream) {
     if (len_dev == nullptr || add == nullptr) return HW_ERR_NULL;
-    if (F < 1 || F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (F < 1 || F > HW_MAX_LAUNCH_FRAGMENTS) return HW_ERR_FRAGMENTS;
     hw::AdvanceArgs a;
     std::memset(&a, 0, sizeof(a));
     a.len_dev = len_dev;
@@ -378,7 +387,7 @@ int hw_validate(const hw_problem* p, int fused) { return validate(p, fused); }
 int hw_plan_debug(const hw_problem* p, int num_cus, hw_plan* plan) {
     // planning needs only the shape and the lengths
     if (p == nullptr || plan == nullptr || p->len == nullptr) return HW_ERR_NULL;
-    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->F < 1 || p->F > HW_MAX_LAUNCH_FRAGMENTS) return HW_ERR_FRAGMENTS;
     if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->Ev < 1 || p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
     for (int f = 0; f < p->F; ++f)
         if (p->len[f] < 0) return HW_ERR_SHAPE;
@@ -391,10 +400,10 @@ static int workspace_bytes_for(const hw_problem* p, int fused, size_t* bytes) {
     int cus = 0;
     int st = device_cus(&cus);
     if (st != HW_OK) return st;
-    hw_plan plan;
-    st = make_plan(p, cus, &plan, fused);
+    CallPlan cp;
+    st = plan_call(p, cus, &cp, fused);
     if (st != HW_OK) return st;
-    *bytes = plan.workspace_bytes;
+    *bytes = cp.workspace_bytes;
     return HW_OK;
 }
 
@@ -412,18 +421,18 @@ int hw_fused_attention_static(const hw_problem* p, void* stream) {
     int cus = 0;
     st = device_cus(&cus);
     if (st != HW_OK) return st;
-    hw_plan plan;
+    CallPlan cp;
     hw_problem q = *p;
-    st = make_plan(&q, cus, &plan);
+    st = plan_call(&q, cus, &cp, 1);
     if (st != HW_OK) return st;
-    if (plan.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES && p->row_blocks == 0 && plan.row_blocks == hw::WIDE_ROW_BLOCKS) {
+    if (cp.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES && p->row_blocks == 0 && cp.plan[0].row_blocks == hw::WIDE_ROW_BLOCKS) {
         // the 128-row workgroups write a partial per split for all rows of a kv head: the 32-row kernel needs a quarter
         // of that with its fewer splits per row group, and the caller left the choice to the library
         q.row_blocks = 2;
-        st = make_plan(&q, cus, &plan);
+        st = plan_call(&q, cus, &cp, 1);
         if (st != HW_OK) return st;
     }
-    if (plan.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES) return HW_ERR_STATIC_SCRATCH;
+    if (cp.workspace_bytes > (size_t)HW_STATIC_SCRATCH_BYTES) return HW_ERR_STATIC_SCRATCH;
     void* ptr = nullptr;
     st = static_scratch(&ptr);
     if (st != HW_OK) return st;

@@ -663,7 +663,7 @@ struct DevHeader {
     const HW_GLOBAL int* len_dev;
     int F, W, Hq, Hkv, S, R;
     int nrg, wgs_per_head, nwg;
-    int prerotated;
+    int slot_stride;
     int flags;
     float sc;
     unsigned magic_gq, magic_s, magic_nrg, magic_wg;

@@ -35,8 +35,10 @@ struct alignas(64) KernelHeader {
                         // min(bound, len_dev[f]) tokens, so a captured launch stays valid while segments grow.
     int F, W, Hq, Hkv, S, R;
     int nrg, wgs_per_head, nwg;
-    int prerotated;
-    int flags;          // KH_XCD_REMAP | KH_DIRECT
+    int slot_stride;    // partial slots per kv head in the workspace: wgs_per_head, or more when the fragments of a call
+                        // are spread over several launches that write side by side (part_o / part_ml then point at this
+                        // launch's first slot)
+    int flags;          // KH_XCD_REMAP | KH_DIRECT | KH_PREROTATED
     float sc;           // scale * log2(e)
     unsigned magic_gq, magic_s, magic_nrg, magic_wg;   // ceil(2^32 / d) for d = Hq/Hkv, S, nrg, wgs_per_head
 };
@@ -44,6 +46,7 @@ static_assert(sizeof(KernelHeader) == 128, "KernelHeader must be 32 dwords");
 constexpr int KH_XCD_REMAP = 1;   // consecutive logical workgroup ids share an XCD (the grid is a multiple of 8)
 constexpr int KH_DIRECT = 2;      // one workgroup per kv head and row group: it normalises its own result and writes out / lse
                                   // itself (part_o then holds the address of out, part_ml that of lse or null); no merge launch
+constexpr int KH_PREROTATED = 4;  // the queries arrive rotated, [F,W,Hq,S,E] (read by the launchers only)
 
 struct KernelArgs {
     KernelHeader h;

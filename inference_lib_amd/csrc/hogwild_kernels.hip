@@ -294,7 +294,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
     size_t orow[RB];
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) orow[rb] = direct ? map_row(a, min(r0 + rb * 16 + n, a.R - 1), hkv, GQ).qrow : 0;
-    store_partials<DT, EV, RB, !EXSEP>(st, ex, wv, n, q, tid, a.part_o, a.part_ml, (size_t)(hkv * a.wgs_per_head + g) * a.R + r0,
+    store_partials<DT, EV, RB, !EXSEP>(st, ex, wv, n, q, tid, a.part_o, a.part_ml, (size_t)(hkv * a.slot_stride + g) * a.R + r0,
                                min(ROWS, a.R - r0), direct, orow);
     HW_MARK(5);
 
@@ -469,7 +469,7 @@ static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, int v
                                dim3(NTHREADS), 0, stream, ka);
         return hipGetLastError();
     }
-    if (ka.h.prerotated) {
+    if (ka.h.flags & KH_PREROTATED) {
         if (ka.h.len_dev != nullptr) return hipErrorInvalidValue;   // device-resident lengths exist for the fused entry only
         if (E == 128) return launch_attention_rb<DT, 128, 128, true, false>(ka, rb, stream);
         return launch_attention_rb<DT, 64, 64, true, false>(ka, rb, stream);

@@ -111,7 +111,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
     a.len_dev = nullptr;
     a.F = ph.F; a.W = ph.LW; a.Hq = ph.Hq; a.Hkv = ph.Hkv; a.S = ph.LS; a.R = rend;
     a.nrg = 1; a.wgs_per_head = ph.nsplit; a.nwg = ph.nwg;
-    a.prerotated = 1; a.flags = 0; a.sc = ph.sc;
+    a.slot_stride = ph.nsplit; a.flags = KH_PREROTATED; a.sc = ph.sc;
     a.magic_gq = ph.magic_gq; a.magic_s = ph.magic_ls; a.magic_nrg = 0; a.magic_wg = 0;
 
     // block-table entry of the token this lane stands for in tile t

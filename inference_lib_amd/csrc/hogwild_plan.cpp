@@ -40,6 +40,8 @@ int validate(const hw_problem* p, int fused) {
     if (p->k == nullptr || p->v == nullptr || p->len == nullptr) return HW_ERR_NULL;
     if (fused && p->RotE > 0 && (p->cosines == nullptr || p->sines == nullptr)) return HW_ERR_NULL;
     if (p->len_dev != nullptr && (!fused || p->RotE != p->E)) return HW_ERR_UNSUPPORTED;   // fused entry, full rotary width only
+    // one launch only: device-resident lengths (a captured step is one attention launch) and the VALU-logits variant
+    if (p->F > HW_MAX_LAUNCH_FRAGMENTS && (p->len_dev != nullptr || p->variant != HW_VARIANT_MFMA)) return HW_ERR_UNSUPPORTED;
     long long rows = (long long)p->W * p->S * (p->Hq / p->Hkv);
     if (rows >= (1 << 20) || p->S >= (1 << 12) || p->Hq / p->Hkv >= (1 << 12)) return HW_ERR_SHAPE;
     if ((long long)p->Hkv * ((rows + 15) / 16) * HW_MAX_SPLITS >= (1 << 20)) return HW_ERR_SHAPE;   // grid size
@@ -63,7 +65,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     if (num_cus < 1) return HW_ERR_SHAPE;
     std::memset(plan, 0, sizeof(*plan));
     // the same limits as validate(): the planner is also reachable on its own (hw_plan_debug)
-    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->F < 1 || p->F > HW_MAX_LAUNCH_FRAGMENTS) return HW_ERR_FRAGMENTS;
     if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->S < 1 || p->Ev < 1 || p->Hq % p->Hkv != 0 || p->len == nullptr) return HW_ERR_SHAPE;
     const long long rows_ll = (long long)p->W * p->S * (p->Hq / p->Hkv);
     if (rows_ll >= (1 << 20) || p->S >= (1 << 12) || p->Hq / p->Hkv >= (1 << 12)) return HW_ERR_SHAPE;
@@ -89,7 +91,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
         tiles += ((long long)p->len[f] + hw::TILE - 1) / hw::TILE;
         if (tiles > (1ll << 30)) return HW_ERR_SHAPE;
     }
-    for (int f = p->F; f <= HW_MAX_FRAGMENTS; ++f) plan->tile_begin[f] = (int)tiles;
+    for (int f = p->F; f <= HW_MAX_LAUNCH_FRAGMENTS; ++f) plan->tile_begin[f] = (int)tiles;
     plan->tiles_per_head = (int)tiles;
 
     // Split-K policy: fill every CU with its resident workgroups once, but at least one tile per wave
@@ -179,6 +181,35 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     return HW_OK;
 }
 
+int plan_call(const hw_problem* p, int num_cus, CallPlan* cp, int fused) {
+    if (cp == nullptr || p == nullptr) return HW_ERR_NULL;
+    std::memset(cp, 0, sizeof(*cp));
+    if (p->F < 1 || p->F > HW_MAX_FRAGMENTS) return HW_ERR_FRAGMENTS;
+    if (p->len == nullptr) return HW_ERR_NULL;
+    cp->groups = (p->F + HW_MAX_LAUNCH_FRAGMENTS - 1) / HW_MAX_LAUNCH_FRAGMENTS;
+    int dummy_rq = 0;
+    for (int i = 0; i < cp->groups; ++i) {
+        // groups of equal size (130 fragments: 44 + 43 + 43, not 64 + 64 + 2)
+        cp->first[i] = (int)(((long long)p->F * i) / cp->groups);
+        cp->count[i] = (int)(((long long)p->F * (i + 1)) / cp->groups) - cp->first[i];
+        hw_problem q = *p;
+        q.F = cp->count[i];
+        q.len = p->len + cp->first[i];
+        q.cap = p->cap != nullptr ? p->cap + cp->first[i] : nullptr;
+        q.rq = &dummy_rq;                      // the room for rotated queries is counted once, below
+        const int st = make_plan(&q, num_cus, &cp->plan[i], fused);
+        if (st != HW_OK) return st;
+        cp->slot_base[i] = cp->slots;
+        cp->slots += cp->plan[i].wgs_per_head;
+    }
+    const size_t rows = (size_t)cp->plan[0].rows;
+    cp->partial_bytes = ((size_t)p->Hkv * cp->slots * rows * ((size_t)p->Ev + 2) * sizeof(float) + 255) & ~(size_t)255;
+    if (fused && p->rq == nullptr && p->RotE != p->E && p->RotE >= 0)
+        cp->rope_bytes = ((size_t)p->F * p->W * p->Hq * p->S * p->E * elem_size(p->dtype) + 255) & ~(size_t)255;
+    cp->workspace_bytes = cp->partial_bytes + cp->rope_bytes;
+    return HW_OK;
+}
+
 int paged_validate(const hw_paged_problem* p) {
     if (p == nullptr) return HW_ERR_NULL;
     if (p->dtype != HW_F32 && p->dtype != HW_F16 && p->dtype != HW_BF16) return HW_ERR_DTYPE;
@@ -208,8 +239,15 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     if (num_cus < 1) return HW_ERR_SHAPE;
     std::memset(plan, 0, sizeof(*plan));
     const bool varlen = p->cu_seqlens_q != nullptr;
+    // the same limits as paged_validate(): the planner is also reachable on its own (hw_paged_plan_debug,
+    // hw_paged_workspace_bytes), and the narrowing below must not be handed anything larger
+    if (p->W < 1 || p->Hq < 1 || p->Hkv < 1 || p->Ev < 1 || p->Hq % p->Hkv != 0) return HW_ERR_SHAPE;
+    if (varlen ? p->total_q < 0 : (p->S < 1 || p->S >= (1 << 12))) return HW_ERR_SHAPE;
+    if (p->block_size < 1 || p->block_size >= (1 << 12) || p->max_blocks < 1) return HW_ERR_SHAPE;
+    if ((long long)p->block_size * p->max_blocks > (1ll << 20)) return HW_ERR_SHAPE;
     const int gq = p->Hq / p->Hkv;
     const long long tokens = varlen ? p->total_q : (long long)p->W * p->S;
+    if (gq >= (1 << 12) || tokens * gq >= (1 << 20) || p->W >= (1 << 20)) return HW_ERR_SHAPE;
     plan->rows = (int)(tokens * gq);
     // rows of one worker share its KV: one 16-row block is enough for plain decoding, two when a worker brings
     // more rows (several query tokens, wide GQA groups)

@@ -394,7 +394,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         for (int rb = 0; rb < RB; ++rb) {
             const float lsum = quarter_sum(st.l[rb]);
             const int row0 = w0 + rb * 16;                            // first row of the block
-            const size_t prow0 = (size_t)(hkv * a.wgs_per_head + g) * a.R + row0;
+            const size_t prow0 = (size_t)(hkv * a.slot_stride + g) * a.R + row0;
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c)              // block c, accumulator rows 4q .. 4q+3 = elements 16c + 4q ..
                 *reinterpret_cast<f32x4*>(stage + n * OSTR + 16 * c + 4 * q) = st.o[rb][c];
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     a.len_dev = nullptr;
     a.F = ph.F; a.W = ph.LW; a.Hq = ph.Hq; a.Hkv = ph.Hkv; a.S = ph.LS; a.R = rend;
     a.nrg = 1; a.wgs_per_head = ph.nsplit; a.nwg = ph.nwg;
-    a.prerotated = 1; a.flags = 0; a.sc = ph.sc;
+    a.slot_stride = ph.nsplit; a.flags = KH_PREROTATED; a.sc = ph.sc;
     a.magic_gq = ph.magic_gq; a.magic_s = ph.magic_ls; a.magic_nrg = 0; a.magic_wg = 0;
 
     // The sequence's block table goes into LDS once: per tile every lane then looks up the block of its own position
@@ -694,7 +694,7 @@ template <class DT>
 static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
     constexpr int NS = 5;
     constexpr int NW = HW_WIDE_WAVES;
-    if (ka.h.prerotated) {
+    if (ka.h.flags & KH_PREROTATED) {
         if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
     } else {

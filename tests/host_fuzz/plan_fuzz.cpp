@@ -38,7 +38,7 @@ static void fuzz_fragments(std::mt19937_64& rng) {
     hw_problem p{};
     const int dts[3] = {HW_F32, HW_F16, HW_BF16};
     p.dtype = dts[U(0, 2)];
-    p.F = (int)U(1, U(0, 3) == 0 ? HW_MAX_FRAGMENTS : 12);
+    p.F = (int)U(1, U(0, 3) == 0 ? HW_MAX_LAUNCH_FRAGMENTS : 12);
     p.Hkv = (int)(U(0, 5) == 0 ? U(1, 64) : (1 << U(0, 3)));
     p.Hq = p.Hkv * (int)(U(0, 9) == 0 ? U(1, 4095) : U(1, 16));
     p.W = (int)(U(0, 9) == 0 ? U(1, 5000) : U(1, 16));
@@ -70,7 +70,7 @@ static void fuzz_fragments(std::mt19937_64& rng) {
         CHECK(plan.tile_begin[f] == tiles, "tile_begin[%d]", f);
         tiles += (len[f] + hw::TILE - 1) / hw::TILE;
     }
-    for (int f = p.F; f <= HW_MAX_FRAGMENTS; ++f) CHECK(plan.tile_begin[f] == tiles, "tile_begin tail %d", f);
+    for (int f = p.F; f <= HW_MAX_LAUNCH_FRAGMENTS; ++f) CHECK(plan.tile_begin[f] == tiles, "tile_begin tail %d", f);
     const int rows = p.W * p.S * (p.Hq / p.Hkv);
     CHECK(plan.rows == rows && plan.tiles_per_head == tiles, "rows / tiles");
     CHECK(plan.row_blocks == 1 || plan.row_blocks == 2 || plan.row_blocks == 8, "row_blocks %d", plan.row_blocks);
@@ -100,6 +100,58 @@ static void fuzz_fragments(std::mt19937_64& rng) {
     CHECK(vs <= 0 && vs >= HW_ERR_STATIC_SCRATCH, "validate status %d", vs);
 }
 
+// A whole call: up to HW_MAX_FRAGMENTS fragments in groups of at most HW_MAX_LAUNCH_FRAGMENTS, one launch each.
+static void fuzz_call(std::mt19937_64& rng) {
+    auto U = [&](long long lo, long long hi) { return (long long)(lo + rng() % (unsigned long long)(hi - lo + 1)); };
+    hw_problem p{};
+    p.dtype = U(0, 1) ? HW_BF16 : HW_F32;
+    p.F = (int)(U(0, 2) == 0 ? U(1, HW_MAX_FRAGMENTS + 2) : U(60, 140));
+    p.Hkv = 1 << U(0, 3);
+    p.Hq = p.Hkv * (int)U(1, 8);
+    p.W = (int)U(1, 70);
+    p.S = (int)U(1, 3);
+    p.E = p.Ev = U(0, 1) ? 128 : 64;
+    p.RotE = U(0, 3) == 0 ? p.E / 2 : p.E;
+    p.scale = 0.1f;
+    p.splits = U(0, 3) == 0 ? (int)U(1, 300) : 0;
+    std::vector<int32_t> len(p.F);
+    for (auto& l : len) l = (int)(U(0, 3) == 0 ? 0 : U(1, 700));
+    p.len = len.data();
+    const int fused = (int)U(0, 1);
+    const int cus = (int)(U(0, 3) == 0 ? U(1, 1024) : 256);
+    CallPlan cp;
+    const int st = plan_call(&p, cus, &cp, fused);
+    if (p.F > HW_MAX_FRAGMENTS) {
+        CHECK(st == HW_ERR_FRAGMENTS, "plan_call took %d fragments (status %d)", p.F, st);
+        return;
+    }
+    if (st != HW_OK) {
+        CHECK(st == HW_ERR_SHAPE, "plan_call status %d", st);
+        return;
+    }
+    CHECK(cp.groups == (p.F + HW_MAX_LAUNCH_FRAGMENTS - 1) / HW_MAX_LAUNCH_FRAGMENTS && cp.groups <= MAX_GROUPS, "groups %d for %d fragments", cp.groups, p.F);
+    int next = 0, slots = 0;
+    for (int i = 0; i < cp.groups; ++i) {
+        CHECK(cp.first[i] == next && cp.count[i] >= 1 && cp.count[i] <= HW_MAX_LAUNCH_FRAGMENTS, "group %d: first %d count %d", i, cp.first[i], cp.count[i]);
+        next += cp.count[i];
+        CHECK(cp.slot_base[i] == slots, "slot base of group %d", i);
+        slots += cp.plan[i].wgs_per_head;
+        long long tiles = 0;
+        for (int f = 0; f < cp.count[i]; ++f) tiles += (len[cp.first[i] + f] + hw::TILE - 1) / hw::TILE;
+        CHECK(cp.plan[i].tiles_per_head == tiles, "tiles of group %d", i);
+        CHECK(cp.plan[i].rows == cp.plan[0].rows && cp.plan[i].row_blocks == cp.plan[0].row_blocks, "groups disagree on the rows");
+    }
+    CHECK(next == p.F && slots == cp.slots, "groups cover %d of %d fragments, %d of %d slots", next, p.F, slots, cp.slots);
+    const size_t need = (size_t)p.Hkv * cp.slots * cp.plan[0].rows * ((size_t)p.Ev + 2) * sizeof(float);
+    const size_t rope = (fused && p.RotE != p.E) ? (size_t)p.F * p.W * p.Hq * p.S * p.E * (p.dtype == HW_F32 ? 4 : 2) : 0;
+    CHECK(cp.partial_bytes >= need && cp.partial_bytes % 256 == 0 && cp.rope_bytes >= rope && cp.workspace_bytes == cp.partial_bytes + cp.rope_bytes,
+          "workspace %zu (partials %zu need %zu, rope %zu need %zu)", cp.workspace_bytes, cp.partial_bytes, need, cp.rope_bytes, rope);
+    if (cp.groups == 1) {      // a call of one launch is the plan of that launch
+        hw_plan plan;
+        CHECK(make_plan(&p, cus, &plan, fused) == HW_OK && plan.workspace_bytes == cp.workspace_bytes && plan.wgs_per_head == cp.slots, "single group differs from make_plan");
+    }
+}
+
 static void fuzz_paged(std::mt19937_64& rng) {
     auto U = [&](long long lo, long long hi) { return (long long)(lo + rng() % (unsigned long long)(hi - lo + 1)); };
     hw_paged_problem p{};
@@ -125,13 +177,16 @@ static void fuzz_paged(std::mt19937_64& rng) {
     const int cus = (int)(U(0, 3) == 0 ? U(1, 1024) : 256);
     hw_paged_plan plan;
     const int st = paged_plan(&p, cus, &plan);
+    {   // sizes beyond the kernels' index ranges are refused by the planner itself
+        const long long tk = varlen ? p.total_q : (long long)p.W * p.S;
+        if (tk * (p.Hq / p.Hkv) >= (1 << 20) || p.W >= (1 << 20)) CHECK(st == HW_ERR_SHAPE, "paged_plan took %lld rows, %d sequences (status %d)", tk * (p.Hq / p.Hkv), p.W, st);
+    }
     if (st != HW_OK) {
         CHECK(st == HW_ERR_SHAPE, "paged_plan status %d", st);
         return;
     }
     const int gq = p.Hq / p.Hkv;
     const long long tokens = varlen ? p.total_q : (long long)p.W * p.S;
-    if (tokens * gq >= (1 << 20)) return;   // paged_validate refuses these before the planner is asked
     CHECK(plan.rows == tokens * gq, "rows");
     CHECK(plan.splits >= 1 && plan.splits <= 64, "splits %d", plan.splits);
     CHECK(plan.row_groups >= 1, "row groups");
@@ -152,6 +207,7 @@ int main(int argc, char** argv) {
     std::mt19937_64 rng(seed);
     for (long i = 0; i < iters; ++i) {
         fuzz_fragments(rng);
+        fuzz_call(rng);
         fuzz_paged(rng);
     }
     // a divisor the multiply-high division gets wrong must be refused: 40 000 decode sequences on 8 kv heads

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
     for name in declared:
         assert hasattr(L.lib, name), name
-    assert L.lib.hw_version() == 4
+    assert L.lib.hw_version() == 5 == L.HW_ABI_VERSION
 
 
 def test_calibration_kernels_live_in_their_own_library():
@@ -96,7 +96,10 @@ def test_validation_happens_on_the_host():
     assert v(_problem(L, scale=-1.0)) == -3
     assert v(_problem(L, E=96, Ev=96, RotE=96)) == -4       # valid but not instantiated: a hard error, never silent
     assert v(_problem(L, Ev=64)) == -4
-    assert v(_problem(L, F=65)) == -5
+    assert v(_problem(L, F=65)) == 0                        # beyond one launch's 64 fragments: several launches
+    assert v(_problem(L, F=512)) == 0 and v(_problem(L, F=513)) == -5
+    assert v(_problem(L, F=65, len_dev=0x1000)) == -4       # device-resident lengths: one launch only
+    assert v(_problem(L, F=65, variant=1)) == -4
     assert v(_problem(L, F=0)) == -5
     assert v(_problem(L, out=None)) == -1
     assert v(_problem(L, cosines=None)) == -1
@@ -229,7 +232,7 @@ def test_paged_validation_happens_on_the_host():
     assert v(_paged(L)) == 0
     assert L.lib.hw_paged_validate(None) == -1
     assert v(_paged(L, dtype=5)) == -2
-    assert v(_paged(L, F=0)) == -5 and v(_paged(L, F=65)) == -5
+    assert v(_paged(L, F=0)) == -5 and v(_paged(L, F=65)) == 0 and v(_paged(L, F=513)) == -5
     assert v(_paged(L, Hq=41)) == -3
     assert v(_paged(L, scale=0.0)) == -3 and v(_paged(L, scale=float("nan"))) == -3
     assert v(_paged(L, block_size=0)) == -3 and v(_paged(L, block_size=4096)) == -3

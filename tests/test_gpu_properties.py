@@ -101,7 +101,19 @@ def test_rows_that_see_nothing_and_empty_fragments(oracle):
     assert_close("rq incl. the empty fragment", rq, rq_ref, 3.2e-2)
 
 
+def _many_fragments(dtype, F, W, S, Hq, Hkv, E, seed, rot_dim=None):
+    """F short fragments (some empty, some longer than a tile), every worker seeing all of them in its own order."""
+    from inference_lib_amd import cases
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(0, 71, (F,), generator=g).tolist()
+    lens[F // 3] = 150
+    lens[-1] = 33
+    orders = [list(torch.randperm(F, generator=g).tolist()) for _ in range(W)]
+    return cases.build_case(f"many{F}_{dtype}", dtype, W, S, Hq, Hkv, E, 1e4, lens, orders, g, rot_dim=rot_dim)
+
+
 def test_fragment_limit(oracle):
+    """64 fragments fill one launch; the call takes up to 512 (the reference's limit, src/binding.cu:79-82)."""
     from inference_lib_amd import _lib, cases
     lens = [40] + [3 + (i % 5) for i in range(63)]
     W = 63
@@ -113,12 +125,75 @@ def test_fragment_limit(oracle):
     assert_close("out", out, o_ref, TOL["bf16"])
     assert_close("lse", lse, l_ref, TOL["bf16"])
     with pytest.raises(_lib.HogwildError) as ei:
-        cd = c.to(_dev())
-        loc = torch.cat([cd.locations, cd.locations[:1]]).contiguous()
-        cs = torch.cat([cd.cos, cd.cos[:1]]).contiguous()
-        _lib.Problem(q=cd.q, locations=loc, keys=cd.keys + cd.keys[:1], values=cd.values + cd.values[:1], scale=c.scale,
-                     out=torch.empty_like(out), cosines=cs, sines=cs)
+        c513 = _many_fragments("bf16", 513, 1, 1, 2, 1, 64, 9).to(_dev())
+        _lib.Problem(q=c513.q, locations=c513.locations, keys=c513.keys, values=c513.values, scale=c513.scale,
+                     out=torch.empty_like(c513.q), cosines=c513.cos, sines=c513.sin)
     assert ei.value.status == -5
+
+
+@pytest.mark.parametrize("dtype,F,W,S,Hq,Hkv,E", [
+    ("bf16", 130, 4, 1, 8, 2, 128),      # three launches of 44 / 43 / 43 fragments, 16 rows per kv head
+    ("f32", 65, 3, 2, 6, 2, 64),         # two launches, fp32
+    ("f16", 129, 8, 2, 32, 2, 128),      # 256 rows per kv head: every launch runs the 128-row kernel
+    ("bf16", 512, 2, 1, 4, 2, 64),       # the limit: eight launches
+])
+def test_more_fragments_than_one_launch_takes(oracle, dtype, F, W, S, Hq, Hkv, E):
+    """More than 64 fragments: groups of at most 64 per attention launch, their split-K partials side by side in the
+    workspace, one merge over all of them.  Checked against the oracle, rotated queries included, and against the same
+    call with the fragments' order reversed (other groups, other partials, same mathematics)."""
+    from inference_lib_amd import _lib
+    c = _many_fragments(dtype, F, W, S, Hq, Hkv, E, seed=F)
+    print(f"case {c.name} F={F} W={W} S={S} Hq={Hq} Hkv={Hkv} E={E}", flush=True)
+    out, lse, rq = run_fused(c.to(_dev()))
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("rq", rq, rq_ref, 1e-5 if dtype == "f32" else 3.2e-2)
+    assert_close("out", out, o_ref, TOL[dtype])
+    assert_close("lse", lse, l_ref, TOL[dtype])
+    cd = c.to(_dev())
+    rev = lambda t: torch.flip(t, dims=[0]).contiguous()
+    out2 = torch.full_like(out, float("nan"))
+    lse2 = torch.full_like(lse, float("nan"))
+    pr = _lib.Problem(q=cd.q, locations=rev(cd.locations), keys=cd.keys[::-1], values=cd.values[::-1], scale=c.scale, out=out2,
+                      cosines=rev(cd.cos), sines=rev(cd.sin), lse=lse2)
+    pr.run()
+    torch.cuda.synchronize()
+    assert_close("out (reversed)", out2, o_ref, TOL[dtype])
+    assert_close("lse (reversed)", lse2, l_ref, TOL[dtype])
+    # the two stages separately give the same bits as the one call
+    out3 = torch.full_like(out, float("nan"))
+    lse3 = torch.full_like(lse, float("nan"))
+    p3 = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=c.scale, out=out3, cosines=cd.cos,
+                      sines=cd.sin, lse=lse3)
+    p3.run(stages=1)
+    p3.run(stages=2)
+    torch.cuda.synchronize()
+    assert torch.equal(out.view(torch.uint8), out3.view(torch.uint8)) and torch.equal(lse.view(torch.uint8), lse3.view(torch.uint8))
+
+
+def test_more_fragments_pre_rotated_and_partial_rotary(oracle):
+    """The other two ways into the attention kernel with more than 64 fragments: hw_sdpa (queries rotated per fragment by
+    the caller) and a rotary width below the head dimension (rotated by the standalone kernel into the workspace)."""
+    from inference_lib_amd import _lib
+    c = _many_fragments("bf16", 100, 3, 1, 6, 2, 128, seed=77)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    rq = torch.full((c.F, W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    _lib.rope(cd.q, cd.cos, cd.sin, rq)
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    _lib.Problem(q=rq, locations=cd.locations, keys=cd.keys, values=cd.values, scale=c.scale, out=out, lse=lse, prerotated=True).run()
+    torch.cuda.synchronize()
+    o2, l2 = oracle.sdpa_fragments(np64(rq), c.locations.numpy(), [np64(k) for k in c.keys], [np64(v) for v in c.values], c.scale)
+    assert_close("sdpa out", out, o2, TOL["bf16"])
+    assert_close("sdpa lse", lse, l2, TOL["bf16"])
+    c = _many_fragments("f16", 70, 2, 2, 4, 2, 64, seed=78, rot_dim=32)
+    out, lse, rq = run_fused(c.to(_dev()))
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("rq", rq, rq_ref, 3.2e-2)
+    assert_close("out", out, o_ref, TOL["f16"])
+    assert_close("lse", lse, l_ref, TOL["f16"])
+    out2, lse2, _ = run_fused(c.to(_dev()), with_rq=False)     # rotated queries go to the workspace instead
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
 
 
 def test_long_fragment_many_tiles_per_workgroup(oracle):
