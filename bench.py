@@ -106,16 +106,50 @@ def time_graph(stream, step_fn, K, warmup=20, min_replays=MIN_REPLAYS, min_total
     return {"median": per[len(per) // 2], "p10": pct(per, 0.10), "p90": pct(per, 0.90), "replays": replays, "graph_steps": n}
 
 
-def load_traffic(key):
+def load_traffic(key, with_commit=False):
     """HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE and WRITE_SIZE in separate runs, each scaled by
     what the same counter reads for the copy kernel of known size this script launches); None when the workload was
-    not measured.  The numbers live next to the rocprof summaries they come from."""
+    not measured.  The numbers live next to the rocprof summaries they come from, each with the commit of the kernel
+    sources it was taken at."""
     try:
         with open(TRAFFIC_JSON) as fh:
             entry = json.load(fh).get(key)
-        return None if entry is None else int(entry["traffic_bytes"])
+        if entry is None:
+            return (None, None) if with_commit else None
+        return (int(entry["traffic_bytes"]), entry.get("commit")) if with_commit else int(entry["traffic_bytes"])
     except (OSError, ValueError, KeyError):
+        return (None, None) if with_commit else None
+
+
+def torch_op_leg(run, stream, K, warmup):
+    """The operator a caller of the reference invokes, torch.ops.libhogatt.hogwild_fused (it sizes and allocates its
+    split-K workspace from torch's caching allocator on every call): per-call time in a Python loop on one stream,
+    synchronised at both ends, and of the same calls captured in a HIP graph.  Cold ring like everything else."""
+    import torch
+    from inference_lib_amd import attention
+    if not attention.HAVE_TORCH_OPS:
         return None
+    cd, case = run.cd, run.case
+    frag = torch.tensor(case.lens, dtype=torch.int32, device=cd.q.device)
+
+    def op(i):
+        keys, vals = run.ring[i % run.n]
+        torch.ops.libhogatt.hogwild_fused(run.out, run.rq, case.scale, cd.locations, cd.q, frag, keys, vals, cd.cos, cd.sin)
+
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            op(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            op(i)
+        torch.cuda.synchronize()
+        loop_us = (time.perf_counter() - t0) / K * 1e6
+    graph = time_graph(stream, op, K, warmup=warmup, min_replays=10, min_total=1000)
+    return {"python_loop": round(loop_us, 3), "hip_graph": round(graph["median"], 3),
+            "what": "torch.ops.libhogatt.hogwild_fused (writes the rotated queries, allocates its workspace per call); "
+                    "python_loop = K calls on one stream between two synchronisations, host-bound; hip_graph = the same calls "
+                    "captured once and replayed"}
 
 
 def bench_lib():
@@ -372,6 +406,7 @@ def main():
     step = time_graph(stream, run.step, K, warmup=Wm)            # the headline: attention + merge, cold ring
     kern = time_graph(stream, run.kernel, K, warmup=Wm)          # the attention kernel alone (merge stage off)
     hot = time_graph(stream, run.hot, K, warmup=Wm, min_replays=10, min_total=1000)
+    torch_op = torch_op_leg(run, stream, K, Wm) if run.rq is not None else None
 
     # ---------------- the same steps with the fragment lengths read from device memory ----------------
     len_dev = torch.tensor(case.lens, dtype=torch.int32, device=dev)
@@ -461,6 +496,7 @@ def main():
             "unit": "GB/s",
             "frac": round(achieved / PEAK_HBM_GBS, 4),
             "traffic": load_traffic(f"attention_kernel/{case.name}"),
+            "traffic_commit": load_traffic(f"attention_kernel/{case.name}", with_commit=True)[1],
             "kernel": "hw::attention_wide_kernel" if run.plan.row_blocks == 8 else "hw::attention_kernel",
             "kernel_us_avg": round(kern["median"], 3),
             "kernel_us_p10_p90": [round(kern["p10"], 3), round(kern["p90"], 3)],
@@ -474,6 +510,7 @@ def main():
             "steps_per_graph": step["graph_steps"],
             "pct_of_peak": round(100.0 * value / PEAK_HBM_GBS, 2),
             "eager_loop_us_per_step": round(eager_us, 3),
+            "torch_op_us_per_step": torch_op,
             "hot_cache_us_per_step": round(hot["median"], 3),
             "device_lengths_us_per_step": round(devlen["median"], 3),
             "hot_cache_GBps": round(kv_bytes / (hot["median"] * 1e-6) / 1e9, 1),

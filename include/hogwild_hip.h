@@ -88,7 +88,7 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   splits     0 = choose automatically; otherwise the number of workgroups per kv head
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
  *              spread over more workgroups that read the same KV); 8 = 128-row workgroups whose waves share every K/V
- *              tile through LDS (16-bit types without len_dev; the automatic choice beyond 64 rows per kv head)
+ *              tile through LDS (16-bit types without len_dev; the automatic choice beyond 96 rows per kv head)
  *   variant    HW_VARIANT_MFMA (0, default): logits and output on the matrix cores.  HW_VARIANT_VALU_QK: the logits
  *              K.Q^T by VALU dot products (v_dot2_f32_bf16 / _f16, v_fma_f32) in the same kernel, the inner product the
  *              reference uses (src/kernels/kernel_v21.cuh:161-180); exists so that the matrix-core choice can be measured
@@ -224,7 +224,11 @@ typedef struct hw_paged_problem {
     void* workspace;
     size_t workspace_bytes;
     int32_t splits;            /* 0 = automatic; otherwise workgroups per (kv head, row group) */
-    int32_t row_blocks;        /* 0 = automatic; 1, 2 or 8 = 16-row MFMA blocks per workgroup (8: 128-row workgroups, 16-bit types, max_blocks <= 8192) */
+    int32_t row_blocks;        /* 0 = automatic; 1, 2 or 8 = 16-row MFMA blocks per workgroup (8: 128-row workgroups, 16-bit types,
+                                  max_blocks <= 8192; the automatic choice beyond 96 query rows per sequence and kv head --
+                                  for packed queries, whose lengths are device data, beyond 96 on average over the
+                                  sequences: a batch of one long and many one-token sequences stays on the 32-row kernel
+                                  unless the caller sets 8) */
 } hw_paged_problem;
 
 typedef struct hw_paged_plan {

@@ -31,15 +31,6 @@
 
 namespace hw {
 
-// tile buffers per wave of the two-row-block 16-bit kernels (tuning knob)
-#ifndef HW_PF2
-#define HW_PF2 2
-#endif
-// waves per SIMD the two-row-block 16-bit kernels are register-budgeted for (tuning knob)
-#ifndef HW_MINW2
-#define HW_MINW2 1
-#endif
-
 // Phase timestamps for kernel tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
 #ifdef HW_CLOCKS
 __device__ unsigned long long hw_clock_buf[4096 * 16];
@@ -452,7 +443,7 @@ static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t 
         hipLaunchKernelGGL((attention_kernel<DT, E, EV, 1, half ? 2 : 1, half ? 2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
                            stream, ka);
     else
-        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, half ? HW_MINW2 : 1, half ? HW_PF2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg),
+        hipLaunchKernelGGL((attention_kernel<DT, E, EV, 2, 1, half ? 2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg),
                            dim3(NTHREADS), 0, stream, ka);
     return hipGetLastError();
 }

@@ -686,14 +686,12 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
 // Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
 // usual cure for a loop that waits) double what the waves read out of LDS per tile, and the kernel got slower by a
 // tenth (27.3 against 24.7 us at 128 rows x 16 K tokens x 8 kv heads, fp16).
-#ifndef HW_WIDE_WAVES
-#define HW_WIDE_WAVES 4
-#endif
+constexpr int WIDE_WAVES = 4;
 
 template <class DT>
 static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
     constexpr int NS = 5;
-    constexpr int NW = HW_WIDE_WAVES;
+    constexpr int NW = WIDE_WAVES;
     if (ka.h.flags & KH_PREROTATED) {
         if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);

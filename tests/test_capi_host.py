@@ -23,6 +23,12 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(L.lib, name), name
     assert L.lib.hw_version() == 5 == L.HW_ABI_VERSION
+    # constants the ctypes mirror repeats
+    for name in ("HW_ABI_VERSION", "HW_MAX_FRAGMENTS", "HW_MAX_LAUNCH_FRAGMENTS", "HW_MAX_SPLITS"):
+        m = re.search(rf"#define\s+{name}\s+(\d+)", header)
+        assert m and int(m.group(1)) == getattr(L, name), name
+    m = re.search(r"#define\s+HW_STATIC_SCRATCH_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", header)
+    assert m and int(m.group(1)) << int(m.group(2)) == L.HW_STATIC_SCRATCH_BYTES
 
 
 def test_calibration_kernels_live_in_their_own_library():

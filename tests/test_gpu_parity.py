@@ -40,6 +40,22 @@ def test_baseline_configs(oracle, idx):
     print(f"  max err out {e1:.3e} lse {e2:.3e}", flush=True)
 
 
+@pytest.mark.parametrize("dtype,W,S", [("f16", 1, 1), ("f16", 4, 1), ("bf16", 2, 3), ("f16", 8, 1), ("f32", 2, 1)])
+def test_the_reference_kernels_compiled_shape(oracle, dtype, W, S):
+    """E = Ev = 128 with 16 query heads per kv head is the one shape the reference's kernel is instantiated for
+    (src/kernels/kernel_v21.cuh:982); here through the fused entry with 16, 64, 96 and 128 rows per kv head (one and two
+    row blocks, several row groups, the 128-row kernel) and in fp32."""
+    from inference_lib_amd import cases
+    lens = tuple([300] + [70 + 9 * w for w in range(W)])
+    c = cases.small_case(dtype=dtype, W=W, S=S, Hq=32, Hkv=2, E=128, lens=lens, seed=51)
+    print(f"case {c.name} W={W} S={S} rows per kv head {W * S * 16}", flush=True)
+    out, lse, rq = run_fused(c.to(_dev()))
+    o_ref, l_ref, rq_ref = oracle_fused(oracle, c)
+    assert_close("rq", rq, rq_ref, 1e-5 if dtype == "f32" else 3.2e-2)
+    assert_close("out", out, o_ref, TOL[dtype])
+    assert_close("lse", lse, l_ref, TOL[dtype])
+
+
 @pytest.mark.parametrize("dtype,E", [("bf16", 128), ("f16", 64), ("f32", 64), ("f32", 128)])
 def test_rope_and_sdpa_entries(oracle, dtype, E):
     """hw_rope and hw_sdpa (pre-rotated queries), the two halves the reference also exports separately

@@ -19,7 +19,6 @@ def test_planner_and_validators_under_sanitizers(tmp_path, seed):
            os.path.join(ROOT, "inference_lib_amd", "csrc", "hogwild_plan.cpp"), "-o", exe]
     subprocess.run(cmd, check=True)
     env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:abort_on_error=0", UBSAN_OPTIONS="print_stacktrace=1")
-    env.pop("LD_PRELOAD", None)
     r = subprocess.run([exe, "1500", str(seed)], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0, r.stdout[-3000:] + r.stderr[-3000:]
     assert "0 failures" in r.stdout

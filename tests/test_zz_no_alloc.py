@@ -121,3 +121,43 @@ def test_static_scratch_refuses_what_does_not_fit():
         pr.run_static()
     assert ei.value.status == -9
     assert "HW_STATIC_SCRATCH_BYTES" in str(ei.value)
+
+
+def test_static_scratch_entry_allocates_nothing_and_can_be_captured(oracle):
+    """What the entry point exists for: on a warmed library it takes no device memory (the driver's free-byte count does
+    not move over a series of calls), and it can run under stream capture (an allocation there would fail the capture):
+    every replay of the captured call gives the eager call's bits."""
+    from inference_lib_amd import _lib, cases
+    c = cases.small_case(dtype="bf16", W=4, S=1, Hq=20, Hkv=4, E=128, lens=(700, 300, 257, 64, 129), seed=7)
+    cd = c.to(_dev())
+    W, Hq, S, E = cd.q.shape
+    out = torch.full((W, Hq, S, E), float("nan"), dtype=cd.q.dtype, device=_dev())
+    lse = torch.full((W, Hq, S), float("nan"), dtype=torch.float32, device=_dev())
+    pr = _lib.Problem(q=cd.q, locations=cd.locations, keys=cd.keys, values=cd.values, scale=cd.scale, out=out,
+                      cosines=cd.cos, sines=cd.sin, lse=lse)
+    pr.run_static()                                      # first call on this device: takes the array's address
+    torch.cuda.synchronize()
+    eager_o, eager_l = out.clone(), lse.clone()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(20):
+        pr.run_static()
+    torch.cuda.synchronize()
+    free1, _ = torch.cuda.mem_get_info()
+    assert free1 == free0, f"device memory moved by {free0 - free1} bytes over 20 calls"
+    assert torch.equal(out, eager_o) and torch.equal(lse, eager_l)
+
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            pr.run_static()
+        for rep in range(3):
+            out.fill_(float("nan"))
+            lse.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager_o) and torch.equal(lse, eager_l), f"replay {rep} differs from the eager call"
+    o_ref, l_ref, _ = oracle_fused(oracle, c)
+    assert_close("out", out, o_ref, TOL[c.dtype])
+    assert_close("lse", lse, l_ref, TOL[c.dtype])
