@@ -389,6 +389,20 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             sacc[rb][tb] = acc;
         }
     }
+    // The V^T operands out of the LDS image, requested here: the LDS answers while the exponentials are taken, and the
+    // output products below then issue back to back.  (Read where they are used, one chunk's pair of reads at a time into
+    // the same registers, every chunk waited for the LDS round trip in front of its two products: eight exposed round
+    // trips per tile.)
+    [[maybe_unused]] u32x4 vops[VLDS ? G::NOC : 1];
+    if constexpr (VLDS) {
+#pragma unroll
+        for (int c = 0; c < G::NOC; ++c) {
+            const char* vp = vimg + voff[c];
+            const u32x2 a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
+            vops[c] = u32x4{a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    }
     // Online softmax with a lazily updated reference: exponentials are taken against st.m, which only moves when
     // a row's maximum exceeds it by more than 2^LAZY_LOG2 (then O and l of that row are rescaled).  Most tiles
     // therefore leave the accumulators alone: no rescale multiplies, and O can stay in the MFMA accumulator
@@ -451,9 +465,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
         if constexpr (VLDS) {
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c) {
-                const char* vp = vimg + voff[c];
-                const u32x2 a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
-                const u32x4 vop = {a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
+                const u32x4 vop = vops[c];
 #pragma unroll
                 for (int rb = 0; rb < RB; ++rb) st.o[rb][c] = Elem<DT>::mfma(vop, pp[rb], st.o[rb][c]);
             }

@@ -152,13 +152,8 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
             maxlim = max(maxlim, pad ? 0 : lim[rb]);
             minlim = min(minlim, lim[rb]);
         }
-#pragma unroll
-        for (int off = 1; off < 16; off <<= 1) {
-            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
-            minlim = min(minlim, __shfl_xor(minlim, off, 64));
-        }
-        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
-        minlim = __builtin_amdgcn_readfirstlane(minlim);
+        maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
+        minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
 
         // Issue the loads of tile t given its table entries: the same number of load instructions whether or not
         // the tile exists (a tile beyond the visible range re-reads one row that is visible, or, if nothing is

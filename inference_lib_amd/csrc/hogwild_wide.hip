@@ -329,13 +329,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
             maxlim = max(maxlim, pad ? 0 : lim[rb]);
             minlim = min(minlim, lim[rb]);
         }
-#pragma unroll
-        for (int off = 1; off < 16; off <<= 1) {
-            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
-            minlim = min(minlim, __shfl_xor(minlim, off, 64));
-        }
-        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
-        minlim = __builtin_amdgcn_readfirstlane(minlim);
+        maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
+        minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
         if (PRE || !staged) {
 #pragma unroll
             for (int i = 1; i < D; ++i) request(i, lt0 + i);
@@ -572,13 +567,8 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
             maxlim = max(maxlim, pad ? 0 : lim[rb]);
             minlim = min(minlim, lim[rb]);
         }
-#pragma unroll
-        for (int off = 1; off < 16; off <<= 1) {
-            maxlim = max(maxlim, __shfl_xor(maxlim, off, 64));
-            minlim = min(minlim, __shfl_xor(minlim, off, 64));
-        }
-        maxlim = __builtin_amdgcn_readfirstlane(maxlim);
-        minlim = __builtin_amdgcn_readfirstlane(minlim);
+        maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
+        minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
         // what the WORKGROUP can see decides which positions are fetched and where its tile loop ends (every wave must
         // take part in every tile's barrier); what the wave can see decides which tiles it multiplies
         int wgmax = 0;
