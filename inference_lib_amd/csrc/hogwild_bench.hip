@@ -13,11 +13,20 @@ typedef unsigned int u32;
 typedef u32 u32x4 __attribute__((ext_vector_type(4)));
 
 __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4* src, size_t n16, u32* sink) {
+    // eight independent 16-byte loads per thread and round (a wave has 8 KB in flight), so that a launch with one
+    // workgroup per compute unit is bound by memory and not by one load's latency per round
+    constexpr int UN = 8;
     u32x4 acc = {0, 0, 0, 0};
-    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) {
-        u32x4 x = __builtin_nontemporal_load(src + i);
-        acc ^= x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    for (; i + (UN - 1) * stride < n16; i += UN * stride) {
+        u32x4 x[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) x[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) acc ^= x[u];
     }
+    for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
     u32 r = acc.x ^ acc.y ^ acc.z ^ acc.w;
     if (r == 0x9e3779b9u) sink[threadIdx.x] = r;   // practically never: keeps the loads alive without a store stream
 }
