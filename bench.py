@@ -462,6 +462,9 @@ def main():
     nbare = max(2, big.numel() // kvb16)
     bare = time_graph(stream, lambda i: _lib.check(blib.hw_stream_read(big.data_ptr() + (i % nbare) * kvb16, kvb16, sink.data_ptr(),
                                                                        C.c_void_p(stream.cuda_stream)), "hw_stream_read"), K, **small)
+    cus = _lib.lib.hw_device_cus()
+    bare_shape = time_graph(stream, lambda i: _lib.check(blib.hw_stream_read_shaped(big.data_ptr() + (i % nbare) * kvb16, kvb16, sink.data_ptr(), cus,
+                                                                                    C.c_void_p(stream.cuda_stream)), "hw_stream_read_shaped"), K, **small)
     del big
 
     graph_us = step["median"]
@@ -516,6 +519,8 @@ def main():
             "hot_cache_GBps": round(kv_bytes / (hot["median"] * 1e-6) / 1e9, 1),
             "stream_read_GBps": round(stream_gbs, 1),
             "bare_read_us_per_launch": {"bytes": kvb16, "us": round(bare["median"], 3)},
+            "bare_read_in_launch_shape_us": {"bytes": kvb16, "workgroups": cus, "us": round(bare_shape["median"], 3),
+                                             "what": "the same bytes read by one 256-thread workgroup per compute unit, the attention kernel's launch shape"},
             "rope_append_us_per_call": round(append["median"], 3),
             "build_inputs_us_per_call": round(build["median"], 3),
             "append_plus_attention_us_per_layer": round(layer_t["median"], 3),
