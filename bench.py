@@ -65,6 +65,8 @@ def parse_args():
     ap.add_argument("--layers", type=int, default=64, help="stack workload: decoder layers")
     ap.add_argument("--seq-len", type=int, default=12528, help="paged workload: tokens per sequence")
     ap.add_argument("--block-size", type=int, default=16, help="paged workload: tokens per cache block")
+    ap.add_argument("--q-lens", default="1,8,32,64", help="varlen workload: query tokens of the four sequences")
+    ap.add_argument("--row-blocks", type=int, default=0, help="paged workloads: 16-row blocks per workgroup (0 = the planner's choice; 8 = the 128-row kernel)")
     return ap.parse_args()
 
 
@@ -578,7 +580,8 @@ def bench_paged(args, dev, quick=False):
     varlen = args.workload == "varlen"
     cu = None
     if varlen:   # packed queries: the last 1 / 8 / 32 / 64 positions of the four sequences (causal)
-        q_lens = [1, 8, 32, 64]
+        q_lens = [int(x) for x in args.q_lens.split(",")]
+        assert len(q_lens) == W and all(0 <= n <= L for n in q_lens), "--q-lens takes four lengths"
         T = sum(q_lens)
         cu = torch.tensor([0] + [sum(q_lens[:i + 1]) for i in range(W)], dtype=torch.int32, device=dev)
         q = torch.randn((F, T, Hq, D), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -599,13 +602,13 @@ def bench_paged(args, dev, quick=False):
         bt = perm[i * W * nblk:(i + 1) * W * nblk].reshape(W, nblk).contiguous().to(dev)
         tables.append(bt)
         pr = _lib.PagedProblem(q=q, locations=loc, fragment_lengths=fl, key_cache=kc, value_cache=vc, block_table=bt,
-                               scale=scale, out=out, lse=lse, splits=args.splits, cu_seqlens_q=cu)
+                               scale=scale, out=out, lse=lse, splits=args.splits, cu_seqlens_q=cu, row_blocks=args.row_blocks)
         if ws is None:
             ws = torch.empty(pr.workspace_bytes(), dtype=torch.uint8, device=dev)
         pr.set_workspace(ws)
         problems.append(pr)
     plan = _lib.paged_plan(W=W, Hq=Hq, Hkv=Hkv, Ev=D, block_size=bs, max_blocks=nblk, num_cus=_lib.lib.hw_device_cus(), S=S,
-                           splits=args.splits, total_q=(q.size(1) if varlen else None))
+                           splits=args.splits, total_q=(q.size(1) if varlen else None), row_blocks=args.row_blocks)
     K, Wm = args.steps, args.warmup
     if getattr(args, "profile_steps", 0) > 0 and not quick:
         profile_mode(args, dev, torch.cuda.Stream(), lambda i: problems[i % nring].run(), kv_bytes, "paged " + args.workload)
@@ -641,7 +644,7 @@ def bench_paged(args, dev, quick=False):
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": K, "warmup": Wm,
         "ms_per_step": round(graph_us * 1e-3, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": (f"varlen paged: W={W} sequences x {L} tokens, query tokens per sequence 1/8/32/64, " if varlen else
+        "config": {"workload": (f"varlen paged: W={W} sequences x {L} tokens, query tokens per sequence {args.q_lens.replace(',', '/')}, " if varlen else
                                 f"paged decode: W={W} sequences x {L} tokens, S={S}, ") + f"Hq={Hq} Hkv={Hkv} D={D} bf16, block_size={bs}, F={F}", "kv_bytes_per_step": kv_bytes, "cold_cache_ring_sets": nring,
                    "workgroups": plan.workgroups, "splits": plan.splits},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",

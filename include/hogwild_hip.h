@@ -40,7 +40,7 @@
 extern "C" {
 #endif
 
-#define HW_ABI_VERSION 5
+#define HW_ABI_VERSION 6
 #define HW_MAX_FRAGMENTS 512          /* fragments per call, the reference's limit (src/binding.cu:79-82) */
 #define HW_MAX_LAUNCH_FRAGMENTS 64    /* fragments one attention launch takes (their table travels in the kernel arguments);
                                          a call with more runs ceil(F / 64) attention launches, whose split-K partials lie
@@ -237,6 +237,10 @@ typedef struct hw_paged_plan {
     int32_t row_groups;        /* over all workers; an upper bound for the variable-length operator */
     int32_t splits;            /* workgroups per (kv head, row group); tile t of a sequence goes to wave t mod (4 * splits) */
     int32_t workgroups;
+    int32_t device_planned;    /* packed queries in 128-row workgroups: the split is decided on the device from the query and KV
+                                  lengths, in the prologue of the attention kernel.  row_groups is then the number
+                                  of workgroup slots per kv head (each takes a row group's share of tiles, or nothing),
+                                  splits = 1 */
     size_t workspace_bytes;
 } hw_paged_plan;
 

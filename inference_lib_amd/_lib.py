@@ -17,7 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libhogwild_hip.so")
 
 HW_MAX_FRAGMENTS = 512          # per call
 HW_MAX_LAUNCH_FRAGMENTS = 64    # per attention launch (what hw_plan describes)
-HW_ABI_VERSION = 5              # the version the structures below mirror
+HW_ABI_VERSION = 6              # the version the structures below mirror
 HW_MAX_SPLITS = 256
 HW_STATIC_SCRATCH_BYTES = 8 << 20
 HW_F32, HW_F16, HW_BF16 = 0, 1, 2
@@ -77,7 +77,7 @@ class HwPagedProblem(C.Structure):
 class HwPagedPlan(C.Structure):
     _fields_ = [
         ("rows", C.c_int32), ("row_blocks", C.c_int32), ("row_groups", C.c_int32), ("splits", C.c_int32),
-        ("workgroups", C.c_int32), ("workspace_bytes", C.c_size_t),
+        ("workgroups", C.c_int32), ("device_planned", C.c_int32), ("workspace_bytes", C.c_size_t),
     ]
 
 

@@ -151,6 +151,8 @@ int run(const hw_problem* p, void* stream_, int fused, int stages = HW_STAGE_ATT
     ma.W = p->W; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = p->S; ma.R = rows;
     ma.wgs_per_head = cp.slots;
     ma.xcd_local = (cp.groups == 1 && plan0.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
+    ma.row_tab = nullptr;
+    ma.pslots = 0;
     e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
     return (int)e;
 }
@@ -182,8 +184,12 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     ph.vcache = p->value_cache;
     ph.block_table = p->block_table;
     ph.cu_q = p->cu_seqlens_q;
+    // partial sums by (split, row), or -- planned on the device -- by workgroup slot, then the merge's row table
+    const bool planned = plan.device_planned != 0;
+    const size_t prows = planned ? (size_t)plan.row_groups * hw::PLAN_SLOT_ROWS : (size_t)plan.splits * plan.rows;
     ph.part_o = reinterpret_cast<float*>(p->workspace);
-    ph.part_ml = ph.part_o + (size_t)p->Hkv * plan.splits * plan.rows * p->Ev;
+    ph.part_ml = ph.part_o + (size_t)p->Hkv * prows * p->Ev;
+    int* row_tab = reinterpret_cast<int*>(ph.part_ml + (size_t)p->Hkv * prows * 2);
     ph.F = p->F; ph.W = p->W; ph.Hq = p->Hq; ph.Hkv = p->Hkv;
     ph.LW = varlen ? p->total_q : p->W;
     ph.LS = varlen ? 1 : p->S;
@@ -193,7 +199,7 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     ph.nitems = plan.row_groups;
     ph.nrg = varlen ? 1 : plan.row_groups / p->W;
     ph.nwg = plan.workgroups;
-    ph.xcd_remap = (plan.workgroups % 8 == 0) ? 1 : 0;
+    ph.flags = ((plan.workgroups % 8 == 0) ? hw::PH_XCD_REMAP : 0) | (planned ? hw::PH_PLANNED : 0);
     ph.sc = (float)((double)p->scale * 1.4426950408889634074);
     ph.magic_gq = magic(p->Hq / p->Hkv);
     ph.magic_ls = magic(ph.LS);
@@ -218,6 +224,9 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     ma.wgs_per_head = plan.splits;
     // a variable-length launch may leave row groups of the grid unused, and with them parts of an XCD's share
     ma.xcd_local = (!varlen && plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
+    ma.row_tab = planned ? row_tab : nullptr;
+    ma.pslots = planned ? plan.row_groups : 0;
+    if (planned) ma.wgs_per_head = 8;       // a row's slots are device data: the merge shape that suits a handful of them
     e = hw::launch_merge(ma, p->dtype, p->Ev, stream);
     return (int)e;
 }

@@ -695,7 +695,7 @@ struct PagedDevHeader {
     int R;
     int block_size, max_blocks, num_blocks;
     int nsplit, nitems, nrg, nwg;
-    int xcd_remap;
+    int flags;
     float sc;
     unsigned magic_gq, magic_ls, magic_bs, magic_nsplit, magic_nitems, magic_nrg;
 };

@@ -61,6 +61,11 @@ struct MergeArgs {
     float* lse;
     int W, Hq, Hkv, S, R, wgs_per_head;
     int xcd_local;      // kv head h was computed on XCD h / (Hkv/8): merge it there
+    // Partials laid out by workgroup slot instead of by row (the paged launch that is planned on the device, see
+    // PagedHeader): row_tab[r] = {first slot | slots << 16, row within the slot}, a slot holds PLAN_SLOT_ROWS rows, pslots
+    // slots per kv head; wgs_per_head then only bounds the slots of a row (for the choice of the merge kernel's shape).
+    const int* row_tab;
+    int pslots;
 };
 
 hipError_t launch_attention(const KernelArgs& ka, int dtype, int E, int rb, int variant, hipStream_t stream);
@@ -83,8 +88,8 @@ struct alignas(64) PagedHeader {
     const void* vcache;        // [num_blocks, Hkv, block_size, Ev]
     const int* block_table;    // [W, max_blocks]
     const int* cu_q;           // [W + 1] query-token prefix sums, or null: worker w owns tokens w*LS .. (w+1)*LS-1
-    float* part_o;             // [Hkv][nsplit][R][Ev]
-    float* part_ml;            // [Hkv][nsplit][R][2]
+    float* part_o;             // [Hkv][nsplit][R][Ev]; planned on the device: [Hkv][nitems][PLAN_SLOT_ROWS][Ev]
+    float* part_ml;            // [Hkv][nsplit][R][2];  planned: [Hkv][nitems][PLAN_SLOT_ROWS][2], the merge's row table right behind it
     int F, W, Hq, Hkv, LW, LS;
     int R;                     // LW*LS*(Hq/Hkv): query rows per kv head
     int block_size, max_blocks, num_blocks;
@@ -92,12 +97,18 @@ struct alignas(64) PagedHeader {
     int nitems;                // row groups over all workers (an upper bound when cu_q is given)
     int nrg;                   // row groups per worker (fixed-length operator)
     int nwg;
-    int xcd_remap;
+    int flags;                 // PH_*
     float sc;                  // scale * log2(e)
     unsigned magic_gq, magic_ls, magic_bs, magic_nsplit, magic_nitems, magic_nrg;   // ceil(2^32 / d)
     int pad[8];
 };
 static_assert(sizeof(PagedHeader) == 192, "PagedHeader must be 48 dwords");
+constexpr int PH_XCD_REMAP = 1;    // consecutive logical workgroup ids share an XCD
+// The launch is planned on the device (packed queries in 128-row workgroups): nsplit = 1, nitems = workgroup slots per
+// kv head, and what slot j of a head does -- which row group of which sequence, which share of its tiles -- every
+// workgroup works out for itself from the query and KV lengths (plan_slot).  Behind part_ml the workgroups of kv head 0
+// leave the merge kernel a table of where each row's partial sums lie (MergeArgs::row_tab).
+constexpr int PH_PLANNED = 2;
 
 struct CopyBlocksArgs {
     const void* key_states;    // [B, Hkv, S_new, E]   (element strides below, innermost contiguous)

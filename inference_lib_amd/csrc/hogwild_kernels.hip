@@ -338,11 +338,24 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     const int rr = pg / GPR, pgl = pg % GPR;               // row within the workgroup, partial group within the row
     const bool live = rblk * RPW + rr < a.R;
     const int r = live ? rblk * RPW + rr : a.R - 1;        // (a row that does not exist re-reads the last one and stores nothing)
-    const int ns = a.wgs_per_head;
+    int ns = a.wgs_per_head;
     const float* ml = a.part_ml + ((size_t)hkv * ns * a.R + r) * 2;
-    const size_t mstride = (size_t)a.R * 2;
+    size_t mstride = (size_t)a.R * 2;
     const float* po = a.part_o + ((size_t)hkv * ns * a.R + r) * EV + e4 * 4;
-    const size_t ostride = (size_t)a.R * EV;
+    size_t ostride = (size_t)a.R * EV;
+    if (a.row_tab != nullptr) {     // partials by workgroup slot: this row's are in slots first .. first + ns - 1, at row `rl` of each
+        // (clamped: the table is device data, and a malformed prefix array of query lengths leaves rows that no entry
+        // was written for)
+        const int x = a.row_tab[2 * r];
+        const int rl = min(max(a.row_tab[2 * r + 1], 0), PLAN_SLOT_ROWS - 1);
+        ns = min(max(x >> 16, 0), a.pslots);
+        const int first = min(x & 0xffff, a.pslots - ns);
+        const size_t base = ((size_t)hkv * a.pslots + first) * PLAN_SLOT_ROWS + rl;
+        ml = a.part_ml + base * 2;
+        mstride = (size_t)PLAN_SLOT_ROWS * 2;
+        po = a.part_o + base * EV + e4 * 4;
+        ostride = (size_t)PLAN_SLOT_ROWS * EV;
+    }
 
     float m_run = NEG_BIG, l_run = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};

@@ -80,7 +80,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
 
     // logical workgroup id = ((kv head * nitems) + item) * nsplit + split; consecutive ids share an XCD
     int bid = blockIdx.x;
-    if (ph.xcd_remap) bid = (bid & 7) * (ph.nwg >> 3) + (bid >> 3);
+    if (ph.flags & PH_XCD_REMAP) bid = (bid & 7) * (ph.nwg >> 3) + (bid >> 3);
     const int hi = fast_div(bid, ph.magic_nsplit);
     const int split = bid - hi * ph.nsplit;
     const int hkv = fast_div(hi, ph.magic_nitems);

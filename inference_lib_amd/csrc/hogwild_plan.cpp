@@ -253,10 +253,13 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     // more rows (several query tokens, wide GQA groups)
     const long long rows_per_worker = varlen ? (tokens * gq + p->W - 1) / p->W : (long long)p->S * gq;
     plan->row_blocks = rows_per_worker <= 16 ? 1 : 2;
-    // many rows per sequence: 128-row workgroups whose waves share every K/V tile through LDS (16-bit types; the kernel
-    // keeps a sequence's block table in LDS, up to PAGED_WIDE_MAX_BLOCKS entries)
+    // more than one 16-row block per sequence: workgroups of up to 128 rows whose waves share every K/V tile through LDS
+    // (16-bit types; the kernel keeps a sequence's block table in LDS, up to PAGED_WIDE_MAX_BLOCKS entries).  Measured on
+    // four sequences of 12 528 tokens with 3 / 6 / 12 / 19 query tokens each (15 ... 95 rows per sequence): 36.7 / 36.7 /
+    // 45.9 / 69.4 us against 49.4 / 49.5 / 84.6 / 84.7 us of the 32-row workgroups, which stream a sequence's KV once per
+    // 32 rows; with one token each (5 rows) the two are equal (36.0 / 36.1 us).
     const bool wide_ok = p->dtype != HW_F32 && p->max_blocks <= hw::PAGED_WIDE_MAX_BLOCKS;
-    if (wide_ok && rows_per_worker > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
+    if (wide_ok && rows_per_worker > 16) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
     if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
@@ -266,6 +269,35 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     else items = (long long)p->W * (((long long)p->S * gq + rpw - 1) / rpw);
     if (items < 1) items = 1;
     plan->row_groups = (int)items;
+    if (wide && varlen && p->splits <= 0 && p->W <= hw::PLAN_MAX_GROUPS && items <= hw::PLAN_MAX_GROUPS) {
+        // Packed queries in 128-row workgroups: how many rows a sequence brings and how long its KV is are device data,
+        // so the device deals the workgroups (every workgroup works out its own share in its prologue):
+        // every kv head gets `slots` workgroup slots -- the CUs filled once, a slot per possible row group at least, not
+        // more than a slot per four tiles of the longest KV the tables allow -- and each row group takes a share of them
+        // in proportion to its work.  A caller that fixes the split (splits > 0) gets the unplanned launch below.
+        const long long tiles = ((long long)p->block_size * p->max_blocks + hw::TILE - 1) / hw::TILE;
+        const long long fill = num_cus / p->Hkv > 0 ? num_cus / p->Hkv : 1;
+        const long long by_work = (long long)p->W * tiles / 4;
+        long long slots = fill < by_work ? fill : by_work;
+        if (slots < items) slots = items;
+        // many possible row groups: the launch oversubscribes the CUs anyway, and slots beyond one per row group are
+        // what lets the device cut a long sequence among many short ones
+        if (2 * items > fill) slots = items + (fill < by_work ? fill : by_work);
+        if (slots >= (1 << 16) || (long long)p->Hkv * slots >= (1 << 20)) return HW_ERR_SHAPE;
+        plan->device_planned = 1;
+        plan->row_groups = (int)slots;
+        plan->splits = 1;
+        plan->workgroups = (int)(p->Hkv * slots);
+        const unsigned long long positions = (unsigned long long)p->block_size * p->max_blocks + hw::TILE;
+        if (!magic_exact((unsigned long long)slots, (unsigned long long)p->Hkv * slots) ||
+            !magic_exact((unsigned long long)gq, (unsigned long long)tokens * gq + 32) ||
+            !magic_exact((unsigned long long)p->block_size, positions))
+            return HW_ERR_SHAPE;
+        plan->workspace_bytes = (size_t)p->Hkv * (size_t)slots * hw::PLAN_SLOT_ROWS * ((size_t)p->Ev + 2) * sizeof(float) +
+                                (size_t)(plan->rows > 0 ? plan->rows : 1) * 2 * sizeof(int);
+        plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
+        return HW_OK;
+    }
     int splits = p->splits;
     if (splits <= 0) {
         // The paged kernels run one workgroup per CU.  Few (kv head, row group) pairs: split until every CU has

@@ -26,6 +26,28 @@
 #include "../../include/hogwild_hip.h"
 #include "hogwild_kernels.h"
 
+namespace hw {
+
+// Phase timestamps of the 128-row kernels for tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
+#ifdef HW_CLOCKS
+__device__ unsigned long long hw_wide_clock_buf[1024 * 4 * 16];
+#define HW_MARK(i)                                                                                  \
+    do {                                                                                            \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
+            hw_wide_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (i)] = wall_clock64();    \
+    } while (0)
+#define HW_NOTE(i, v)                                                                               \
+    do {                                                                                            \
+        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
+            hw_wide_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (i)] = (unsigned long long)(v); \
+    } while (0)
+#else
+#define HW_MARK(i) do { } while (0)
+#define HW_NOTE(i, v) do { } while (0)
+#endif
+
+}  // namespace hw
+
 #include "hogwild_device.h"
 
 namespace hw {
@@ -179,6 +201,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15;
     const int q = lane >> 4;
+    HW_MARK(8);
 
     // the kernel arguments in one burst (see attention_kernel)
     const int fl = lane & (MAXF - 1);
@@ -230,6 +253,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     vtr_lane_offsets<G::VROW>(voff, lane);
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(hb.lo), "+s"(hb.hi) : : "memory");
     const DevHeader a = __builtin_bit_cast(DevHeader, hb);
+    HW_MARK(0);
 
     int bid = blockIdx.x;
     if (a.flags & KH_XCD_REMAP) bid = (bid & 7) * (a.nwg >> 3) + (bid >> 3);
@@ -265,7 +289,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     // range: the same number of transfers, no memory traffic, zeros in LDS
     auto request = [&](int sl, int lt) {
         const unsigned tile_bytes = (unsigned)(lt * TILE * image_row);
-        wide_request<TPW>(view, my_image + sl * SLOT, lt < lt1 ? tile_bytes : OOB_OFFSET, off);
+        wide_request<TPW>(view, __builtin_amdgcn_readfirstlane(my_image + sl * SLOT), lt < lt1 ? tile_bytes : OOB_OFFSET, off);
     };
 
     auto open_segment = [&]() {
@@ -293,9 +317,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     };
     bool more = todo != 0;
     if (more) open_segment();
+    HW_MARK(6);
+    bool hw_first = true;
 
     while (more) {
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
+        if (hw_first) HW_MARK(7);
         if (!PRE && staged) {
             wrot.stage(cs_lds, tid, nws);
             // The barrier above has waited for every load of open_segment: the other look-ahead tiles can be requested
@@ -308,10 +335,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         } else {
             qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
         }
-        if (tid % TPR == 0) lim_lds[tid / TPR] = (r0 + tid / TPR < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;
+        int limv = (r0 + tid / TPR < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;   // by every thread, see paged_wide_kernel
+        asm volatile("" : "+v"(limv));
+        if (tid % TPR == 0) lim_lds[tid / TPR] = limv;
         // q_lds and lim_lds become visible: a barrier for LDS only.  __syncthreads() would also wait for the stores of
         // the rotated queries to be acknowledged by memory, which nobody here depends on.
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        if (hw_first) HW_MARK(1);
 
         // this wave's query operands and mask bounds
         u32x4 qreg[RB * G::KJ];
@@ -348,6 +378,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
                 if (rs >= NS) rs -= NS;
                 request(rs, l + D);
                 asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
+                if (hw_first) { HW_MARK(2); hw_first = false; }
             };
             const int lfast = maxlim > 0 ? min(lt1, minlim / TILE) : lt0;
 #pragma unroll 1
@@ -383,7 +414,9 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     {
         constexpr int OSTR = EV + 4;                                  // floats per staged row (padded against bank conflicts)
         static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+        HW_MARK(3);
         __syncthreads();                                              // every wave has left the last tile
+        HW_MARK(4);
         float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
@@ -406,6 +439,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
             }
         }
     }
+
+    HW_MARK(5);
 
     // rotated queries of zero-length fragments are still part of the operator's visible output
     if (!PRE && a.rq != nullptr && g == 0) {
@@ -430,6 +465,148 @@ __device__ __forceinline__ void lds_transfer_flat(unsigned lds, unsigned long lo
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds), "v"(src) : "m0", "memory");
 }
 #pragma clang diagnostic pop
+
+// The split of a packed-query launch, decided on the device (query lengths and KV lengths are device tensors,
+// src/binding.cu:144-181) -- by every workgroup for itself, in its prologue: the inputs are a few hundred bytes that
+// all workgroups read, and a planning kernel in front of the launch cost 5.8 us plus the gap between two launches.
+// One thread per sequence and then per row group (at most PLAN_MAX_GROUPS of either; the host sends larger batches
+// down the unplanned path).  Every kv head has `pslots` workgroup slots.  A row group = up to 128 rows of one sequence;
+// its work is its sequence's tiles times the cost of a tile (a group of at most 64 rows multiplies one 16-row block per
+// wave instead of two: 0.6 against 0.8 us measured).  Every group takes one slot and a share of the others in
+// proportion to its work (what the rounding leaves over goes to the groups with the most work per slot), four tiles per
+// slot at least; slots are numbered through the groups in order.  Returns what slot `item` does
+// (found = false: nothing), and -- for the workgroups of kv head 0 that hold a group's first slot -- tells the merge
+// kernel through row_tab where the partial sums of the group's rows lie.
+struct PlanSlot {
+    int w, rg, qs, qe, split, ns;
+    bool found;
+};
+__device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, bool first_head, int GQ, int T, int tid) {
+    constexpr int NT = NTHREADS;
+    static_assert(NT == PLAN_MAX_GROUPS && WIDE_ROWS <= NT, "one thread per sequence, per row group, per row of a group");
+    int* sc_a = lds;                     // scan buffers
+    int* sc_b = lds + NT;
+    int* seq_qs = lds + 2 * NT;
+    int* seq_qe = lds + 3 * NT;
+    int* seq_tiles = lds + 4 * NT;
+    int* grp_w = lds + 5 * NT;
+    int* grp_rg = lds + 6 * NT;
+    int* wave_part = lds + 7 * NT;       // [NT / 64]
+    int* shared = lds + 7 * NT + NT / 64;         // total of a scan; then the slot's entry (6 ints)
+    const int lane = tid & 63, wv = tid >> 6;
+    const int pslots = ph.nitems;
+
+    // Inclusive scan of one int per thread over the first `nact` threads (the others hold zero and get nothing useful
+    // back); the sum of all goes to shared[0].
+    auto scan = [&](int v, int nact) {
+        int* src = sc_a;
+        int* dst = sc_b;
+        src[tid] = v;
+        __syncthreads();
+        for (int off = 1; off < nact; off <<= 1) {
+            dst[tid] = src[tid] + (tid >= off ? src[tid - off] : 0);
+            __syncthreads();
+            int* t = src; src = dst; dst = t;
+        }
+        const int r = src[tid];
+        if (tid == nact - 1) shared[0] = r;
+        __syncthreads();
+        return r;
+    };
+    // Sum of one int per thread over the workgroup: DPP within rows of 16 lanes, the four rows of a wave by readlane, the
+    // waves through LDS.
+    auto block_total = [&](int v) {
+        v += row_dpp<0xB1>(v);
+        v += row_dpp<0x4E>(v);
+        v += row_dpp<0x141>(v);
+        v += row_dpp<0x140>(v);
+        const int wt = __builtin_amdgcn_readlane(v, 0) + __builtin_amdgcn_readlane(v, 16) + __builtin_amdgcn_readlane(v, 32) +
+                       __builtin_amdgcn_readlane(v, 48);
+        if (lane == 0) wave_part[wv] = wt;
+        __syncthreads();
+        int s = wave_part[0];
+#pragma unroll
+        for (int i = 1; i < NT / 64; ++i) s += wave_part[i];
+        return s;
+    };
+
+    // sequences: query-token range, row groups, tiles of the KV any fragment may see
+    const int cap = ph.block_size * ph.max_blocks;
+    int cnt = 0;
+    if (tid < ph.W) {
+        const int qs = min(max(ph.cu_q[tid], 0), T);
+        const int qe = min(max(ph.cu_q[tid + 1], qs), T);
+        int len = 0;
+        for (int f = 0; f < ph.F; ++f) len = max(len, ph.frag_len[f * ph.W + tid]);
+        len = min(len, cap);
+        seq_qs[tid] = qs;
+        seq_qe[tid] = qe;
+        seq_tiles[tid] = (len + TILE - 1) / TILE;
+        cnt = ((qe - qs) * GQ + WIDE_ROWS - 1) / WIDE_ROWS;
+    }
+    const int gend = scan(cnt, ph.W);                   // row groups up to and including this sequence
+    for (int g = gend - cnt; g < min(gend, NT); ++g) {  // (a malformed prefix array could ask for more groups than threads)
+        grp_w[g] = tid;
+        grp_rg[g] = g - (gend - cnt);
+    }
+    const int G = min(shared[0], min(NT, pslots));
+    __syncthreads();
+
+    // row groups: work, and the most slots it may take (four tiles per slot at least)
+    int gw = 0, grg = 0, work = 0, most = 1, rows = 0;
+    if (tid < G) {
+        gw = grp_w[tid];
+        grg = grp_rg[tid];
+        rows = min((seq_qe[gw] - seq_qs[gw]) * GQ - grg * WIDE_ROWS, WIDE_ROWS);
+        work = seq_tiles[gw] * (rows > WIDE_ROWS / 2 ? 4 : 3);
+        most = max(1, seq_tiles[gw] / 4);
+    }
+    // One slot each, and the other pslots - G in proportion to the work (rounded down, so they fit; the quotient in
+    // floating point, nudged down so that it never exceeds the exact one).
+    const int all_work = block_total(work);
+    const float share = (float)(pslots - G) * (1.0f - 1.0f / (1 << 20)) * __builtin_amdgcn_rcpf((float)max(all_work, 1));
+    int n = tid < G ? min(1 + (int)((float)work * share), most) : 0;
+    // what the rounding left over (fewer slots than groups) goes, one slot each, to the groups with the most work per slot
+    const int left = pslots - block_total(n);
+    const int load = (tid < G && n < most) ? __float_as_int((float)work * __builtin_amdgcn_rcpf((float)n)) : -1;   // (>= 0: ordered like the floats)
+    sc_a[tid] = load;
+    __syncthreads();
+    int ahead = 0;
+    for (int g = 0; g < G; ++g) ahead += (sc_a[g] > load || (sc_a[g] == load && g < tid)) ? 1 : 0;
+    if (load >= 0 && ahead < left) ++n;
+    __syncthreads();                                    // sc_a is a scan buffer again
+    const int slot0 = scan(n, G) - n;
+    n = max(min(n, pslots - slot0), 0);                 // (cannot bite)
+
+    // the group that owns this workgroup's slot publishes the entry
+    if (tid == 0) shared[1] = -1;
+    __syncthreads();
+    if (tid < G && item >= slot0 && item < slot0 + n) {
+        shared[1] = gw; shared[2] = grg; shared[3] = seq_qs[gw]; shared[4] = seq_qe[gw]; shared[5] = item - slot0; shared[6] = n;
+    }
+    __syncthreads();
+    PlanSlot r;
+    r.w = shared[1]; r.rg = shared[2]; r.qs = shared[3]; r.qe = shared[4]; r.split = shared[5]; r.ns = shared[6];
+    r.found = r.w >= 0;
+    // where the merge finds the partial sums of a row: {first slot | slots << 16, row within the slot}; rows behind the
+    // last sequence have none (the merge writes zeros for them)
+    if (first_head) {
+        HW_GLOBAL int* row_tab = reinterpret_cast<HW_GLOBAL int*>(ph.part_ml + (size_t)ph.Hkv * pslots * PLAN_SLOT_ROWS * 2);
+        if (r.found && r.split == 0) {
+            const int nrows = min((r.qe - r.qs) * GQ - r.rg * WIDE_ROWS, WIDE_ROWS);
+            const int row = r.qs * GQ + r.rg * WIDE_ROWS + tid;
+            if (tid < nrows && row < ph.R) {
+                row_tab[2 * row] = (item - r.split) | (r.ns << 16);
+                row_tab[2 * row + 1] = tid;
+            }
+        }
+        if (item == 0) {
+            const int covered = min(seq_qe[ph.W - 1] * GQ, ph.R);
+            for (int i = covered * 2 + tid; i < ph.R * 2; i += NT) row_tab[i] = 0;
+        }
+    }
+    return r;
+}
 
 // The paged operators (hogwild_paged_sdpa / hogwild_varlen_paged_sdpa, see hogwild_paged.hip) for many query rows per
 // sequence: one workgroup = one kv head x one group of up to 128 rows of ONE sequence x every nsplit-th 32-token tile of
@@ -468,6 +645,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     const int n = lane & 15;
     const int q = lane >> 4;
 
+    HW_MARK(8);
     PagedHeaderBits hb;
     paged_header_request(hb);
     // this wave's share of a tile's transfers: the first half of the waves fill the K image, the second half V
@@ -484,36 +662,52 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : (lslot ^ (2 * vimg_segment_key<G::VROW>(row)))) << 4);
     }
     const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
-    WaveState<RB, G::NOC> st;
-#pragma unroll
-    for (int rb = 0; rb < RB; ++rb) {
-        st.m[rb] = NEG_BIG;
-        st.l[rb] = 0.f;
-#pragma unroll
-        for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    st.fresh = true;
     unsigned voff[G::NOC];                             // this lane's positions in a V image (transposed reads)
     vtr_lane_offsets<G::VROW>(voff, lane);
     const PagedDevHeader ph = paged_header_wait(hb);
+    HW_MARK(0);
 
     // logical workgroup id = ((kv head * nitems) + item) * nsplit + split; consecutive ids share an XCD
     int bid = blockIdx.x;
-    if (ph.xcd_remap) bid = (bid & 7) * (ph.nwg >> 3) + (bid >> 3);
+    if (ph.flags & PH_XCD_REMAP) bid = (bid & 7) * (ph.nwg >> 3) + (bid >> 3);
     const int hi = fast_div(bid, ph.magic_nsplit);
-    const int split = bid - hi * ph.nsplit;
+    int split = bid - hi * ph.nsplit;
     const int hkv = fast_div(hi, ph.magic_nitems);
     const int item = hi - hkv * ph.nitems;
     const int GQ = ph.Hq / ph.Hkv;
-
-    const PagedItem it = paged_item<WIDE_ROWS>(ph, item, lane, GQ);
-    if (!it.found) return;                  // the grid is sized for the worst case; uniform over the workgroup
-    const int w = it.w, rg = it.rg, qs = it.qs, qe = it.qe;
     const int T = ph.LW * ph.LS;
+
+    // Which rows of which sequence, and which share of its tiles.  A launch planned on the device (PH_PLANNED) says so in
+    // the slot table behind the partial sums, one entry per workgroup slot of a kv head; otherwise the item is a row
+    // group in the order of the sequences, every one with the same nsplit workgroups.
+    int w, rg, qs, qe, ns;
+    size_t pbase;                           // row of the partial arrays that holds the workgroup's first row
+    if (ph.flags & PH_PLANNED) {
+        const PlanSlot ps = plan_slot(ph, reinterpret_cast<int*>(ring), item, hkv == 0, GQ, T, tid);   // (the ring is not in use yet)
+        if (!ps.found) return;              // a slot the plan left empty; uniform over the workgroup
+        w = __builtin_amdgcn_readfirstlane(ps.w);
+        rg = __builtin_amdgcn_readfirstlane(ps.rg);
+        qs = __builtin_amdgcn_readfirstlane(ps.qs);
+        qe = __builtin_amdgcn_readfirstlane(ps.qe);
+        split = __builtin_amdgcn_readfirstlane(ps.split);
+        ns = __builtin_amdgcn_readfirstlane(ps.ns);
+        pbase = (size_t)(hkv * ph.nitems + item) * PLAN_SLOT_ROWS;
+    } else {
+        const PagedItem it = paged_item<WIDE_ROWS>(ph, item, lane, GQ);
+        if (!it.found) return;              // the grid is sized for the worst case; uniform over the workgroup
+        w = it.w, rg = it.rg, qs = it.qs, qe = it.qe;
+        ns = ph.nsplit;
+        pbase = (size_t)(hkv * ph.nsplit + split) * ph.R + (size_t)qs * GQ + (size_t)rg * WIDE_ROWS;
+    }
+    HW_MARK(6);
+    HW_NOTE(9, (w << 20) | (rg << 12) | (split << 6) | ns);
     const int r0 = qs * GQ + rg * WIDE_ROWS;    // first row of the workgroup (global numbering: token * GQ + head in group)
     const int rend = qe * GQ;                   // end of the worker's rows
     if (r0 >= rend) return;                     // uniform over the workgroup
-    const int w0 = r0 + wv * WROWS;             // first row of this wave
+    // A group of at most 64 rows (a short sequence, or the tail of a long one) is dealt 16 rows per wave instead of 32:
+    // every wave then has one 16-row block to multiply per tile instead of one wave two and the others none, and the
+    // workgroup's tile time, which the busiest wave sets, is that of one block.
+    const bool light = rend - r0 <= 16 * NW;    // uniform over the workgroup
     const int cap = ph.block_size * ph.max_blocks;
     const HW_GLOBAL int* btw = ph.block_table + (size_t)w * ph.max_blocks;
     const unsigned long long image = reinterpret_cast<unsigned long long>(k_wave ? ph.kcache : ph.vcache);
@@ -541,136 +735,170 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         for (int i = tid; i < nent; i += NT) bt_lds[i] = btw[i];
     }
 
-    for (int f = 0; f < ph.F; ++f) {
-        QueryRotation<DT, E, WIDE_ROWS, G::QSTR, true, NT> qrot;
-        qrot.load(a, f, hkv, r0, GQ, tid);
-        const int lm = ph.loc[(size_t)f * T + fast_div(min(r0 + tid / TPR, rend - 1), ph.magic_gq)];
-        const int flen = ph.frag_len[ph.cu_q != nullptr ? f * ph.W + w : f];
-
-        __syncthreads();   // the previous fragment's readers are done with q_lds / lim_lds / the ring
-        qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tid);
-        if (tid % TPR == 0) lim_lds[tid / TPR] = (r0 + tid / TPR < rend) ? max(0, min(min(flen, cap), lm < cap ? lm + 1 : cap)) : 0x7fffffff;
-        __syncthreads();
-
-        u32x4 qreg[RB * G::KJ];
+    // Everything from here on exists twice, for two and for one 16-row block per wave.  The branch is taken once per
+    // workgroup and the two copies share nothing but the values above, so each keeps the registers of its own tile loops.
+    auto run = [&](auto rbx) {
+        constexpr int RBX = decltype(rbx)::value;
+        constexpr int wrows = 16 * RBX;             // rows per wave
+        const int w0 = r0 + wv * wrows;             // first row of this wave
+        WaveState<RBX, G::NOC> st;
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb)
+        for (int rb = 0; rb < RBX; ++rb) {
+            st.m[rb] = NEG_BIG;
+            st.l[rb] = 0.f;
 #pragma unroll
-            for (int j = 0; j < G::KJ; ++j)
-                qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * WROWS + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
-        int lim[RB];
-        int maxlim = 0, minlim = 0x7fffffff;
-#pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            lim[rb] = lim_lds[wv * WROWS + rb * 16 + n];
-            const bool pad = w0 + rb * 16 + n >= rend;
-            maxlim = max(maxlim, pad ? 0 : lim[rb]);
-            minlim = min(minlim, lim[rb]);
+            for (int c = 0; c < G::NOC; ++c) st.o[rb][c] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-        maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
-        minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
-        // what the WORKGROUP can see decides which positions are fetched and where its tile loop ends (every wave must
-        // take part in every tile's barrier); what the wave can see decides which tiles it multiplies
-        int wgmax = 0;
-#pragma unroll
-        for (int i = 0; i < WIDE_ROWS / 64; ++i) {
-            const int r = i * 64 + lane;
-            wgmax = max(wgmax, r0 + r < rend ? lim_lds[r] : 0);
-        }
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) wgmax = max(wgmax, __shfl_xor(wgmax, off, 64));
-        wgmax = __builtin_amdgcn_readfirstlane(wgmax);
+        st.fresh = true;
 
-        // Source addresses of this wave's share of tile t (TPW transfers): every lane looks up the block of the row it
-        // fetches in each transfer.  A position beyond what the workgroup can see is replaced by the last visible one, so a
-        // tile that does not exist costs the same number of transfers and no new memory traffic to speak of, and no byte
-        // outside the visible part of the sequence is read.
-        auto addresses = [&](unsigned long long* src, int t) {
-#pragma unroll
-            for (int j = 0; j < TPW; ++j) {
-                const int tok = min(t * TILE + trow[j], wgmax - 1);
-                const int bi = fast_div(tok, ph.magic_bs);
-                const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
-                const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
-                src[j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
-            }
-        };
-        auto request = [&](int sl, const unsigned long long* src) {
-#pragma unroll
-            for (int j = 0; j < TPW; ++j) lds_transfer_flat(my_image + sl * SLOT + j * 1024, src[j]);
-        };
+        for (int f = 0; f < ph.F; ++f) {
+            QueryRotation<DT, E, WIDE_ROWS, G::QSTR, true, NT> qrot;
+            qrot.load(a, f, hkv, r0, GQ, tid);
+            const int lm = ph.loc[(size_t)f * T + fast_div(min(r0 + tid / TPR, rend - 1), ph.magic_gq)];
+            const int flen = ph.frag_len[ph.cu_q != nullptr ? f * ph.W + w : f];
 
-        if (wgmax > 0) {   // uniform over the workgroup
-            // tiles of this workgroup: split, split + nsplit, ...  The addresses of a request are formed one tile earlier
-            // (after the barrier, next to the arithmetic): the request at the top of a tile is then four transfers and
-            // nothing else, and no wave reaches the barrier late because it was still looking up blocks.
-            const int ns = ph.nsplit;
-            unsigned long long src[TPW];
+            __syncthreads();   // the previous fragment's readers are done with q_lds / lim_lds / the ring
+            if (f == 0) HW_MARK(7);
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tid);
+            // (computed by every thread and pinned there: the compiler waits for a load where its result is first used, and a
+            // use under the condition below leaves the wait to whatever next touches the registers -- inside the tile loops,
+            // where a wait for "all loads" also waits for the look-ahead transfers it does not know of)
+            int limv = (r0 + tid / TPR < rend) ? max(0, min(min(flen, cap), lm < cap ? lm + 1 : cap)) : 0x7fffffff;
+            asm volatile("" : "+v"(limv));
+            if (tid % TPR == 0) lim_lds[tid / TPR] = limv;
+            __syncthreads();
+            if (f == 0) HW_MARK(1);
+
+            {
+                u32x4 qreg[RBX * G::KJ];
 #pragma unroll
-            for (int i = 0; i < D; ++i) {
-                addresses(src, split + i * ns);
-                request(i, src);
-            }
-            addresses(src, split + D * ns);
-            // two loops with one instantiation of the tile arithmetic each (see attention_wide_kernel)
-            int sl = 0;
-            int t = split;
-            auto arrive = [&]() {                         // request tile t + D * ns, wait for tile t, form the next addresses
-                int rs = sl + D;
-                if (rs >= NS) rs -= NS;
-                request(rs, src);
-                // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
-                // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
-                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
-                addresses(src, t + (D + 1) * ns);
-            };
-            const int tfast = maxlim > 0 ? min(minlim, wgmax) / TILE : 0;   // tiles below it are seen completely by every row of the wave
-#pragma unroll 1
-            for (; t < tfast; t += ns) {
-                arrive();
-                const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
-                sl = sl + 1 == NS ? 0 : sl + 1;
-            }
-#pragma unroll 1
-            for (; t * TILE < wgmax; t += ns) {           // uniform over the workgroup: every wave leaves at the same tile
-                arrive();
-                if (t * TILE < maxlim) {
-                    const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                for (int rb = 0; rb < RBX; ++rb)
+#pragma unroll
+                    for (int j = 0; j < G::KJ; ++j)
+                        qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * wrows + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+                int lim[RBX];
+                int maxlim = 0, minlim = 0x7fffffff;
+#pragma unroll
+                for (int rb = 0; rb < RBX; ++rb) {
+                    lim[rb] = lim_lds[wv * wrows + rb * 16 + n];
+                    const bool pad = w0 + rb * 16 + n >= rend;
+                    maxlim = max(maxlim, pad ? 0 : lim[rb]);
+                    minlim = min(minlim, lim[rb]);
                 }
-                sl = sl + 1 == NS ? 0 : sl + 1;
-            }
-            // the requests behind the last tile must have landed before the ring is used again
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-    }
+                maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
+                minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
+                // what the WORKGROUP can see decides which positions are fetched and where its tile loop ends (every wave must
+                // take part in every tile's barrier); what the wave can see decides which tiles it multiplies
+                int wgmax = 0;
+#pragma unroll
+                for (int i = 0; i < WIDE_ROWS / 64; ++i) {
+                    const int r = i * 64 + lane;
+                    wgmax = max(wgmax, r0 + r < rend ? lim_lds[r] : 0);
+                }
+#pragma unroll
+                for (int off = 1; off < 64; off <<= 1) wgmax = max(wgmax, __shfl_xor(wgmax, off, 64));
+                wgmax = __builtin_amdgcn_readfirstlane(wgmax);
 
-    // ---- every wave stores the partial of its own rows, 16-row blocks staged through the ring (see attention_wide_kernel) ----
-    {
-        constexpr int OSTR = EV + 4;
-        static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
-        __syncthreads();
-        float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
+                // Source addresses of this wave's share of tile t (TPW transfers): every lane looks up the block of the row it
+                // fetches in each transfer.  A position beyond what the workgroup can see is replaced by the last visible one, so a
+                // tile that does not exist costs the same number of transfers and no new memory traffic to speak of, and no byte
+                // outside the visible part of the sequence is read.
+                // (block index without the branch of fast_div: a multiplier of 0 stands for "divide by one", and with a
+                // branch per lookup the four table reads of a request wait for each other instead of flying together)
+                const int bs_one = ph.magic_bs == 0 ? -1 : 0;
+                auto addresses = [&](unsigned long long* src, int t) {
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
-            const float lsum = quarter_sum(st.l[rb]);
-            const int row0 = w0 + rb * 16;
-            const size_t prow0 = (size_t)(hkv * ph.nsplit + split) * ph.R + row0;
+                    for (int j = 0; j < TPW; ++j) {
+                        const int tok = min(t * TILE + trow[j], wgmax - 1);
+                        const int bi = (int)__umulhi((unsigned)tok, ph.magic_bs) | (tok & bs_one);
+                        const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
+                        const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
+                        src[j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
+                    }
+                };
+                auto request = [&](int sl, const unsigned long long* src) {
 #pragma unroll
-            for (int c = 0; c < G::NOC; ++c)              // block c, accumulator rows 4q .. 4q+3 = elements 16c + 4q ..
-                *reinterpret_cast<f32x4*>(stage + n * OSTR + 16 * c + 4 * q) = st.o[rb][c];
-            if (q == 0 && row0 + n < rend) *reinterpret_cast<HW_GLOBAL f32x2*>(ph.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
-            const int nvalid = min(16, rend - row0);
-            HW_GLOBAL float* dst = ph.part_o + prow0 * EV;
+                    for (int j = 0; j < TPW; ++j) lds_transfer_flat(__builtin_amdgcn_readfirstlane(my_image + sl * SLOT + j * 1024), src[j]);
+                };
+
+                if (wgmax > 0) {   // uniform over the workgroup
+                    // tiles of this workgroup: split, split + nsplit, ...  The addresses of a request are formed one tile earlier
+                    // (after the barrier, next to the arithmetic): the request at the top of a tile is then four transfers and
+                    // nothing else, and no wave reaches the barrier late because it was still looking up blocks.
+                    unsigned long long src[TPW];
 #pragma unroll
-            for (int ps = 0; ps < 16 * EV / 256; ++ps) {
-                const int idx = ps * 256 + lane * 4;
-                const int rr = idx / EV, e = idx % EV;
-                if (rr < nvalid) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * OSTR + e);
+                    for (int i = 0; i < D; ++i) {
+                        addresses(src, split + i * ns);
+                        request(i, src);
+                    }
+                    addresses(src, split + D * ns);
+                    // two loops with one instantiation of the tile arithmetic each (see attention_wide_kernel)
+                    int sl = 0;
+                    int t = split;
+                    auto arrive = [&]() {                         // request tile t + D * ns, wait for tile t, form the next addresses
+                        int rs = sl + D;
+                        if (rs >= NS) rs -= NS;
+                        request(rs, src);
+                        // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
+                        // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
+                        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
+                        addresses(src, t + (D + 1) * ns);
+                    };
+                    const int tfast = maxlim > 0 ? min(minlim, wgmax) / TILE : 0;   // tiles below it are seen completely by every row of the wave
+#pragma unroll 1
+                    for (; t < tfast; t += ns) {
+                        arrive();
+                        const char* slot = ring + sl * SLOT;
+                        compute_tile<DT, E, EV, RBX, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                        sl = sl + 1 == NS ? 0 : sl + 1;
+                    }
+#pragma unroll 1
+                    for (; t * TILE < wgmax; t += ns) {           // uniform over the workgroup: every wave leaves at the same tile
+                        arrive();
+                        if (t * TILE < maxlim) {
+                            const char* slot = ring + sl * SLOT;
+                            compute_tile<DT, E, EV, RBX, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                        }
+                        sl = sl + 1 == NS ? 0 : sl + 1;
+                    }
+                    // the requests behind the last tile must have landed before the ring is used again
+                    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                }
             }
         }
-    }
+
+        // ---- every wave stores the partial of its own rows, 16-row blocks staged through the ring (see attention_wide_kernel) ----
+        {
+            constexpr int OSTR = EV + 4;
+            static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+            HW_MARK(3);
+            __syncthreads();
+            float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
+            {
+#pragma unroll
+                for (int rb = 0; rb < RBX; ++rb) {
+                    const float lsum = quarter_sum(st.l[rb]);
+                    const int row0 = w0 + rb * 16;
+                    const size_t prow0 = pbase + (size_t)(row0 - r0);
+#pragma unroll
+                    for (int c = 0; c < G::NOC; ++c)              // block c, accumulator rows 4q .. 4q+3 = elements 16c + 4q ..
+                        *reinterpret_cast<f32x4*>(stage + n * OSTR + 16 * c + 4 * q) = st.o[rb][c];
+                    if (q == 0 && row0 + n < rend) *reinterpret_cast<HW_GLOBAL f32x2*>(ph.part_ml + (prow0 + n) * 2) = f32x2{st.m[rb], lsum};
+                    const int nvalid = min(16, rend - row0);
+                    HW_GLOBAL float* dst = ph.part_o + prow0 * EV;
+#pragma unroll
+                    for (int ps = 0; ps < 16 * EV / 256; ++ps) {
+                        const int idx = ps * 256 + lane * 4;
+                        const int rr = idx / EV, e = idx % EV;
+                        if (rr < nvalid) *reinterpret_cast<HW_GLOBAL f32x4*>(dst + idx) = *reinterpret_cast<const f32x4*>(stage + rr * OSTR + e);
+                    }
+                }
+            }
+        }
+        HW_MARK(5);
+    };
+    if (light) run(std::integral_constant<int, 1>{});
+    else run(std::integral_constant<int, RB>{});
 }
 
 // Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
@@ -719,4 +947,10 @@ hipError_t launch_paged_attention_wide(const PagedHeader& ph, int dtype, int E, 
 }
 
 }  // namespace hw
+
+#ifdef HW_CLOCKS
+extern "C" int hw_debug_read_wide_clocks(unsigned long long* host, size_t n) {
+    return (int)hipMemcpyFromSymbol(host, HIP_SYMBOL(hw::hw_wide_clock_buf), n * sizeof(unsigned long long));
+}
+#endif
 

@@ -167,7 +167,7 @@ static void fuzz_paged(std::mt19937_64& rng) {
     p.num_blocks = (int)U(1, 1 << 16);
     p.scale = 0.1f;
     p.splits = U(0, 3) == 0 ? (int)U(1, 80) : 0;
-    p.row_blocks = (int)U(0, 2);
+    p.row_blocks = (int)(U(0, 4) == 0 ? 8 : U(0, 2));
     const bool varlen = U(0, 1);
     int32_t dummy = 0;
     if (varlen) {
@@ -191,7 +191,16 @@ static void fuzz_paged(std::mt19937_64& rng) {
     CHECK(plan.splits >= 1 && plan.splits <= 64, "splits %d", plan.splits);
     CHECK(plan.row_groups >= 1, "row groups");
     CHECK((long long)plan.workgroups == (long long)p.Hkv * plan.row_groups * plan.splits && plan.workgroups < (1 << 20), "workgroups");
-    const size_t need = (size_t)p.Hkv * plan.splits * (size_t)(plan.rows > 0 ? plan.rows : 1) * ((size_t)p.Ev + 2) * sizeof(float);
+    size_t need = (size_t)p.Hkv * plan.splits * (size_t)(plan.rows > 0 ? plan.rows : 1) * ((size_t)p.Ev + 2) * sizeof(float);
+    if (plan.device_planned) {
+        // the device deals `row_groups` workgroup slots per kv head: packed queries in 128-row workgroups only, no fixed
+        // split, a thread of one workgroup per sequence and per possible row group, a slot per possible row group at
+        // least; partial sums by slot, then two ints per row for the merge
+        CHECK(varlen && plan.row_blocks == 8 && p.splits <= 0 && plan.splits == 1, "device-planned launch of the wrong kind");
+        CHECK(p.W <= hw::PLAN_MAX_GROUPS && plan.row_groups < (1 << 16), "device-planned launch too large");
+        CHECK(plan.row_groups >= p.W + tokens * gq / 128, "fewer slots (%d) than possible row groups", plan.row_groups);
+        need = (size_t)p.Hkv * plan.row_groups * hw::PLAN_SLOT_ROWS * ((size_t)p.Ev + 2) * sizeof(float) + (size_t)plan.rows * 2 * sizeof(int);
+    }
     CHECK(plan.workspace_bytes >= need, "workspace");
     check_division((unsigned)plan.splits, (unsigned long long)plan.workgroups - 1, "workgroup id / splits");
     check_division((unsigned)plan.row_groups, (unsigned long long)p.Hkv * plan.row_groups - 1, "(head, item) / items");

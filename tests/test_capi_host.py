@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol():
     assert declared == set(L.EXPORTS), (declared ^ set(L.EXPORTS))
     for name in declared:
         assert hasattr(L.lib, name), name
-    assert L.lib.hw_version() == 5 == L.HW_ABI_VERSION
+    assert L.lib.hw_version() == 6 == L.HW_ABI_VERSION
     # constants the ctypes mirror repeats
     for name in ("HW_ABI_VERSION", "HW_MAX_FRAGMENTS", "HW_MAX_LAUNCH_FRAGMENTS", "HW_MAX_SPLITS"):
         m = re.search(rf"#define\s+{name}\s+(\d+)", header)
@@ -265,10 +265,9 @@ def test_paged_plan_invariants():
     # short sequences: never more waves than tiles at the longest sequence the table allows
     pl = L.paged_plan(W=1, Hq=8, Hkv=8, Ev=128, block_size=16, max_blocks=8, num_cus=256, S=1)
     assert pl.splits == 1
-    # several query tokens per worker: two row blocks, several row groups
+    # more than 16 rows per worker: workgroups of up to 128 rows (16-bit types, at most 8192 table entries per sequence), the CUs filled once
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=12)
-    assert pl.row_blocks == 2 and pl.row_groups == 2 * 2
-    # more than 96 rows per worker: 128-row workgroups (16-bit types, at most 8192 table entries per sequence), the CUs filled once
+    assert pl.row_blocks == 8 and pl.row_groups == 2 * 1 and pl.device_planned == 0
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=64, num_cus=256, S=20)
     assert pl.row_blocks == 8 and pl.row_groups == 2 * 1 and pl.splits == 8 and pl.workgroups == 128   # 32 tiles: four per workgroup at least
     pl = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=128, block_size=1, max_blocks=9000, num_cus=256, S=20)   # table too long for LDS
@@ -281,17 +280,32 @@ def test_paged_plan_invariants():
     # variable length: the row-group count is an upper bound over every way of cutting total_q into W sequences
     pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700, row_blocks=2)
     assert pl.rows == 3500 and pl.row_groups >= 8 + 3500 // 32 and pl.workgroups == 8 * pl.row_groups * pl.splits
+    assert pl.device_planned == 0
+    # ... and in 128-row workgroups the device deals the workgroups: a slot per possible row group at least, the CUs
+    # filled once (more slots when the row groups alone oversubscribe the CUs), partial sums by slot
     pl = L.paged_plan(W=8, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, total_q=700)
-    assert pl.row_blocks == 8 and pl.row_groups >= 8 + 3500 // 128 and pl.workgroups == 8 * pl.row_groups * pl.splits
+    groups = 8 + 3500 // 128
+    assert pl.row_blocks == 8 and pl.device_planned == 1 and pl.splits == 1
+    assert pl.row_groups == groups + 32 and pl.workgroups == 8 * pl.row_groups
+    assert pl.workspace_bytes >= 8 * pl.row_groups * 128 * 130 * 4 + 3500 * 8
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
+    assert pl.row_blocks == 8 and pl.device_planned == 1 and pl.row_groups == 32 and pl.workgroups == 256
+    # short tables: not more slots than there can be work for (four tiles per slot)
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=8, num_cus=256, total_q=105)
+    assert pl.device_planned == 1 and pl.row_groups == 8
+    # a caller that fixes the split, too many sequences for the device-side planner, or few rows per sequence: as before
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105, splits=4)
+    assert pl.row_blocks == 8 and pl.device_planned == 0 and pl.row_groups == 8 and pl.splits == 4 and pl.workgroups == 256
+    pl = L.paged_plan(W=300, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=3000)
+    assert pl.row_blocks == 8 and pl.device_planned == 0
+    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=8)
+    assert pl.row_blocks == 1 and pl.device_planned == 0
     # more (kv head, row group) pairs than half the CUs: about three workgroups per CU on long sequences, no
     # splitting at all on short ones or when the pairs alone oversubscribe the chip that far
     pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105, row_blocks=2)
     assert pl.row_groups == 20 and pl.splits == 5 and 3 * 256 <= pl.workgroups < 4 * 256
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=30, num_cus=256, total_q=105, row_blocks=2).splits == 1
-    assert L.paged_plan(W=64, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=640).splits == 1
-    # the same packed queries in 128-row workgroups: 8 row groups at most, the CUs filled once
-    pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
-    assert pl.row_blocks == 8 and pl.row_groups == 8 and pl.splits == 4 and pl.workgroups == 256
+    assert L.paged_plan(W=64, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=640, row_blocks=2).splits == 1
     # explicit split factor is honoured (capped at 64)
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=5).splits == 5
     assert L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=1024, num_cus=256, S=1, splits=500).splits == 64

@@ -158,11 +158,57 @@ def test_varlen_wide_rows():
     """Packed variable-length queries with many tokens per sequence: 5 .. 1000 rows per kv head and sequence, empty and
     one-token sequences in between, sequences shorter than a tile."""
     c = build_paged("bf16", 1, 6, 10, 2, 128, 16, 60, seq_lens=[900, 50, 9, 430, 64, 777], q_lens=[200, 0, 9, 64, 1, 33], seed=77)
-    check(c)                              # 511 rows / 6 sequences = 85 on average: the planner stays with the 32-row kernel
+    check(c)                              # the split decided on the device
     check(c, row_blocks=8, splits=5)
     check(c, row_blocks=2)                # and the narrow kernel agrees with the same oracle
     c = build_paged("f16", 2, 3, 8, 2, 64, 32, 20, seq_lens=[600, 31, 222], q_lens=[100, 31, 64], seed=3, loc_mode="random")
     check(c, row_blocks=8)
+
+
+def test_varlen_split_decided_on_the_device():
+    """Packed queries in 128-row workgroups (16-bit types, more than 16 rows per sequence on average, at most 256 sequences
+    and possible row groups): every workgroup works out from cu_seqlens_q and the fragment lengths which row group of
+    which sequence it serves and which share of that sequence's tiles.  Sequences of very different KV lengths and query
+    counts, empty ones, groups of exactly 64 / 65 / 128 / 129 rows (one or two 16-row blocks per wave, one or two
+    groups), more sequences than a wave has lanes, against the oracle."""
+    from inference_lib_amd import _lib
+    c = build_paged("bf16", 2, 6, 10, 2, 128, 16, 200, seq_lens=[3000, 40, 700, 64, 1500, 9], q_lens=[64, 1, 0, 30, 7, 9], seed=41)
+    pl = _lib.paged_plan(W=6, Hq=10, Hkv=2, Ev=128, block_size=16, max_blocks=200, num_cus=_lib.lib.hw_device_cus(), total_q=111)
+    assert pl.device_planned == 1 and pl.row_blocks == 8
+    check(c)
+    c = build_paged("f16", 1, 4, 2, 2, 64, 32, 40, seq_lens=[1000, 1200, 300, 1280], q_lens=[64, 65, 128, 129], seed=42, loc_mode="random")
+    check(c)
+    rng = np.random.default_rng(12)
+    W = 200
+    seq = [int(x) for x in rng.integers(9, 400, size=W)]
+    ql = [int(min(s, x)) for s, x in zip(seq, rng.integers(2, 10, size=W))]
+    ql[17] = 0
+    c = build_paged("bf16", 1, W, 8, 2, 64, 16, 25, seq_lens=seq, q_lens=ql, seed=43)
+    pl = _lib.paged_plan(W=W, Hq=8, Hkv=2, Ev=64, block_size=16, max_blocks=25, num_cus=_lib.lib.hw_device_cus(), total_q=sum(ql))
+    assert pl.device_planned == 1
+    check(c)
+    # one long prompt among one-token sequences: the long one gets most of the workgroups
+    seq = [6000] + [int(x) for x in rng.integers(20, 300, size=30)]
+    c = build_paged("bf16", 1, 31, 10, 2, 128, 16, 380, seq_lens=seq, q_lens=[120] + [1] * 30, seed=44)
+    check(c)
+
+
+def test_varlen_tokens_behind_the_last_sequence_give_zeros():
+    """total_q may exceed cu_seqlens_q[-1]: the tokens behind the last sequence belong to none.  The device-planned launch
+    gives them zeros (lse -inf); the other launches leave them unspecified, like the reference, but must get the tokens of
+    the sequences right all the same."""
+    c = build_paged("bf16", 1, 3, 10, 2, 128, 16, 40, seq_lens=[500, 300, 77], q_lens=[40, 9, 33], seed=51)
+    want_o, want_l = oracle_paged(c)
+    pad = 7
+    c2 = dict(c)
+    c2["q"] = torch.cat([c["q"], torch.randn((1, pad, 10, 128)).to(c["q"].dtype)], dim=1)
+    c2["loc"] = torch.cat([c["loc"], torch.full((1, pad), 5, dtype=torch.int32)], dim=1)
+    for kw in (dict(), dict(row_blocks=2), dict(row_blocks=8, splits=3)):
+        out, lse = run_paged(c2, **kw)
+        assert_close("out", out[:-pad], want_o, TOL["bf16"])
+        assert_close("lse", lse[:-pad], want_l, TOL["bf16"])
+        if not kw:
+            assert (out[-pad:] == 0).all() and torch.isneginf(lse[-pad:]).all()
 
 
 def test_paged_wide_small_blocks_and_fallbacks():

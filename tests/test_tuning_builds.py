@@ -15,6 +15,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     ("hogwild_kernels.hip", ["-DHW_CLOCKS"]),
     ("hogwild_kernels.hip", ["-DHW_NO_COMPUTE"]),
     ("hogwild_wide.hip", ["-DHW_NO_COMPUTE"]),
+    ("hogwild_wide.hip", ["-DHW_CLOCKS"]),
 ])
 def test_tuning_switches_still_compile(tmp_path, unit, flags):
     if shutil.which(HIPCC) is None and not os.path.exists(HIPCC):
@@ -24,3 +25,37 @@ def test_tuning_switches_still_compile(tmp_path, unit, flags):
            "-I", os.path.join(ROOT, "include"), *flags, "-c", os.path.join(build.CSRC, unit), "-o", str(tmp_path / "unit.o")]
     r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
     assert r.returncode == 0, r.stderr[-3000:]
+
+
+def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp_path):
+    """The 128-row kernels issue their global->LDS tile transfers from inline assembly and count them by hand
+    (s_waitcnt vmcnt(12) or vmcnt(6): three tiles of four or two transfers may stay in flight).  The compiler does not know of them, and
+    every wait it inserts itself for one of ITS loads inside a tile loop -- vmcnt(0), vmcnt(1): it counts only the loads
+    it knows -- also waits for the look-ahead tiles and empties the pipeline at every tile; it has done so when a load's
+    only use sat under a condition in front of the loop and the wait was left to the next touch of the register.  Checked
+    in the generated code: inside the innermost loops of both kernels no wait for vector memory below the look-ahead."""
+    if shutil.which(HIPCC) is None and not os.path.exists(HIPCC):
+        pytest.skip("no hipcc")
+    import re
+    from inference_lib_amd import build
+    asm = tmp_path / "wide.s"
+    cmd = [HIPCC, f"--offload-arch={build.ARCH}", "-O3", "-std=c++17", "-fno-gpu-rdc", "-munsafe-fp-atomics", "--cuda-device-only",
+           *build.DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-S", os.path.join(build.CSRC, "hogwild_wide.hip"), "-o", str(asm)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-3000:]
+    text = asm.read_text()
+    kernels = re.findall(r"^(_ZN2hw(?:17paged_wide_kernel|21attention_wide_kernel)\S*):", text, re.M)
+    assert len(kernels) >= 12, kernels
+    checked = 0
+    for name in kernels:
+        body = text[text.index(name + ":"):]
+        body = body[:body.index("; -- End function")]
+        parts = re.split(r"\n(\.LBB\d+_\d+):", body)
+        for label, block in zip(parts[1::2], parts[2::2]):
+            if "Depth=2" not in block:
+                continue                                   # not inside a tile loop (the loop over fragments / segments is depth 1)
+            ahead = 6 if "ELi64ELi64" in name else 12      # three tiles of two (head dimension 64) or four transfers per wave
+            for m in re.finditer(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", block):
+                checked += 1
+                assert int(m.group(1)) >= ahead, f"{name} {label}: {m.group(0)} inside a tile loop"
+    assert checked >= 2 * len(kernels)                    # every kernel has its own hand-counted waits there
