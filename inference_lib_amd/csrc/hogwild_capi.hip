@@ -223,7 +223,8 @@ int paged_run(const hw_paged_problem* p, void* stream_, int stages) {
     ma.W = ph.LW; ma.Hq = p->Hq; ma.Hkv = p->Hkv; ma.S = ph.LS; ma.R = plan.rows;
     ma.wgs_per_head = plan.splits;
     // a variable-length launch may leave row groups of the grid unused, and with them parts of an XCD's share
-    ma.xcd_local = (!varlen && plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
+    // (a launch planned on the device keeps every slot of a kv head on the head's XCD whatever the slots do)
+    ma.xcd_local = ((!varlen || planned) && plan.workgroups % 8 == 0 && p->Hkv % 8 == 0) ? 1 : 0;
     ma.row_tab = planned ? row_tab : nullptr;
     ma.pslots = planned ? plan.row_groups : 0;
     if (planned) ma.wgs_per_head = 8;       // a row's slots are device data: the merge shape that suits a handful of them

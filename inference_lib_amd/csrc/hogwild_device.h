@@ -704,7 +704,12 @@ static_assert(offsetof(PagedHeader, pad) == 160, "PagedDevHeader mirrors the use
 
 // n / d for n < 2^20, d < 2^12 with the host-computed multiplier ceil(2^32 / d) mod 2^32: one multiply-high instead
 // of the ~25-instruction integer division sequence.  d == 1 gives the multiplier 0, which stands for "n itself".
-__device__ __forceinline__ int fast_div(int n, unsigned magic) { return magic ? (int)__umulhi((unsigned)n, magic) : n; }
+// Without a branch on purpose: the multiplier is uniform, a branch on it cuts the code around every division into basic
+// blocks, and inside a tile loop the loads on either side then wait for each other instead of flying together.
+__device__ __forceinline__ int fast_div(int n, unsigned magic) {
+    const int by_one = magic == 0 ? -1 : 0;
+    return (int)__umulhi((unsigned)n, magic) | (n & by_one);
+}
 
 // The 40 used dwords of a PagedHeader, fetched from the kernel-argument segment with three scalar loads: requested first
 // thing in the kernel (the argument-independent setup runs while they are in flight), waited for and typed later.

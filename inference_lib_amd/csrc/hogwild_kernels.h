@@ -62,7 +62,7 @@ struct MergeArgs {
     int W, Hq, Hkv, S, R, wgs_per_head;
     int xcd_local;      // kv head h was computed on XCD h / (Hkv/8): merge it there
     // Partials laid out by workgroup slot instead of by row (the paged launch that is planned on the device, see
-    // PagedHeader): row_tab[r] = {first slot | slots << 16, row within the slot}, a slot holds PLAN_SLOT_ROWS rows, pslots
+    // PagedHeader): row_tab[kv head][r] = {first slot | slots << 16, row within the slot}, a slot holds PLAN_SLOT_ROWS rows, pslots
     // slots per kv head; wgs_per_head then only bounds the slots of a row (for the choice of the merge kernel's shape).
     const int* row_tab;
     int pslots;
@@ -106,8 +106,8 @@ static_assert(sizeof(PagedHeader) == 192, "PagedHeader must be 48 dwords");
 constexpr int PH_XCD_REMAP = 1;    // consecutive logical workgroup ids share an XCD
 // The launch is planned on the device (packed queries in 128-row workgroups): nsplit = 1, nitems = workgroup slots per
 // kv head, and what slot j of a head does -- which row group of which sequence, which share of its tiles -- every
-// workgroup works out for itself from the query and KV lengths (plan_slot).  Behind part_ml the workgroups of kv head 0
-// leave the merge kernel a table of where each row's partial sums lie (MergeArgs::row_tab).
+// workgroup works out for itself from the query and KV lengths (plan_slot).  Behind part_ml the workgroups leave the
+// merge kernel a table per kv head of where each row's partial sums lie (MergeArgs::row_tab).
 constexpr int PH_PLANNED = 2;
 
 struct CopyBlocksArgs {

@@ -346,8 +346,9 @@ __global__ __launch_bounds__(256) void merge_kernel(const MergeArgs a) {
     if (a.row_tab != nullptr) {     // partials by workgroup slot: this row's are in slots first .. first + ns - 1, at row `rl` of each
         // (clamped: the table is device data, and a malformed prefix array of query lengths leaves rows that no entry
         // was written for)
-        const int x = a.row_tab[2 * r];
-        const int rl = min(max(a.row_tab[2 * r + 1], 0), PLAN_SLOT_ROWS - 1);
+        const int* tab = a.row_tab + ((size_t)hkv * a.R + r) * 2;
+        const int x = tab[0];
+        const int rl = min(max(tab[1], 0), PLAN_SLOT_ROWS - 1);
         ns = min(max(x >> 16, 0), a.pslots);
         const int first = min(x & 0xffff, a.pslots - ns);
         const size_t base = ((size_t)hkv * a.pslots + first) * PLAN_SLOT_ROWS + rl;

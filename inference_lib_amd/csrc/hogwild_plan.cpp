@@ -294,7 +294,7 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
             !magic_exact((unsigned long long)p->block_size, positions))
             return HW_ERR_SHAPE;
         plan->workspace_bytes = (size_t)p->Hkv * (size_t)slots * hw::PLAN_SLOT_ROWS * ((size_t)p->Ev + 2) * sizeof(float) +
-                                (size_t)(plan->rows > 0 ? plan->rows : 1) * 2 * sizeof(int);
+                                (size_t)p->Hkv * (size_t)(plan->rows > 0 ? plan->rows : 1) * 2 * sizeof(int);
         plan->workspace_bytes = (plan->workspace_bytes + 255) & ~(size_t)255;
         return HW_OK;
     }

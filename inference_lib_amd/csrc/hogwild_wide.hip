@@ -475,13 +475,15 @@ __device__ __forceinline__ void lds_transfer_flat(unsigned lds, unsigned long lo
 // wave instead of two: 0.6 against 0.8 us measured).  Every group takes one slot and a share of the others in
 // proportion to its work (what the rounding leaves over goes to the groups with the most work per slot), four tiles per
 // slot at least; slots are numbered through the groups in order.  Returns what slot `item` does
-// (found = false: nothing), and -- for the workgroups of kv head 0 that hold a group's first slot -- tells the merge
-// kernel through row_tab where the partial sums of the group's rows lie.
+// (found = false: nothing), and -- for the workgroup that holds a group's first slot -- tells the merge kernel through
+// the kv head's row table where the partial sums of the group's rows lie (a table per kv head, although they are all the
+// same: the merge of a head runs on the XCD whose workgroups wrote the head's partial sums and table, and finds both in
+// that XCD's L2).
 struct PlanSlot {
     int w, rg, qs, qe, split, ns;
     bool found;
 };
-__device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, bool first_head, int GQ, int T, int tid) {
+__device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, int hkv, int GQ, int T, int tid) {
     constexpr int NT = NTHREADS;
     static_assert(NT == PLAN_MAX_GROUPS && WIDE_ROWS <= NT, "one thread per sequence, per row group, per row of a group");
     int* sc_a = lds;                     // scan buffers
@@ -590,8 +592,8 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
     r.found = r.w >= 0;
     // where the merge finds the partial sums of a row: {first slot | slots << 16, row within the slot}; rows behind the
     // last sequence have none (the merge writes zeros for them)
-    if (first_head) {
-        HW_GLOBAL int* row_tab = reinterpret_cast<HW_GLOBAL int*>(ph.part_ml + (size_t)ph.Hkv * pslots * PLAN_SLOT_ROWS * 2);
+    {
+        HW_GLOBAL int* row_tab = reinterpret_cast<HW_GLOBAL int*>(ph.part_ml + (size_t)ph.Hkv * pslots * PLAN_SLOT_ROWS * 2) + (size_t)hkv * ph.R * 2;
         if (r.found && r.split == 0) {
             const int nrows = min((r.qe - r.qs) * GQ - r.rg * WIDE_ROWS, WIDE_ROWS);
             const int row = r.qs * GQ + r.rg * WIDE_ROWS + tid;
@@ -683,7 +685,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     int w, rg, qs, qe, ns;
     size_t pbase;                           // row of the partial arrays that holds the workgroup's first row
     if (ph.flags & PH_PLANNED) {
-        const PlanSlot ps = plan_slot(ph, reinterpret_cast<int*>(ring), item, hkv == 0, GQ, T, tid);   // (the ring is not in use yet)
+        const PlanSlot ps = plan_slot(ph, reinterpret_cast<int*>(ring), item, hkv, GQ, T, tid);   // (the ring is not in use yet)
         if (!ps.found) return;              // a slot the plan left empty; uniform over the workgroup
         w = __builtin_amdgcn_readfirstlane(ps.w);
         rg = __builtin_amdgcn_readfirstlane(ps.rg);
@@ -803,14 +805,11 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
                 // fetches in each transfer.  A position beyond what the workgroup can see is replaced by the last visible one, so a
                 // tile that does not exist costs the same number of transfers and no new memory traffic to speak of, and no byte
                 // outside the visible part of the sequence is read.
-                // (block index without the branch of fast_div: a multiplier of 0 stands for "divide by one", and with a
-                // branch per lookup the four table reads of a request wait for each other instead of flying together)
-                const int bs_one = ph.magic_bs == 0 ? -1 : 0;
                 auto addresses = [&](unsigned long long* src, int t) {
 #pragma unroll
                     for (int j = 0; j < TPW; ++j) {
                         const int tok = min(t * TILE + trow[j], wgmax - 1);
-                        const int bi = (int)__umulhi((unsigned)tok, ph.magic_bs) | (tok & bs_one);
+                        const int bi = fast_div(tok, ph.magic_bs);
                         const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
                         const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
                         src[j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];

@@ -199,7 +199,7 @@ static void fuzz_paged(std::mt19937_64& rng) {
         CHECK(varlen && plan.row_blocks == 8 && p.splits <= 0 && plan.splits == 1, "device-planned launch of the wrong kind");
         CHECK(p.W <= hw::PLAN_MAX_GROUPS && plan.row_groups < (1 << 16), "device-planned launch too large");
         CHECK(plan.row_groups >= p.W + tokens * gq / 128, "fewer slots (%d) than possible row groups", plan.row_groups);
-        need = (size_t)p.Hkv * plan.row_groups * hw::PLAN_SLOT_ROWS * ((size_t)p.Ev + 2) * sizeof(float) + (size_t)plan.rows * 2 * sizeof(int);
+        need = (size_t)p.Hkv * plan.row_groups * hw::PLAN_SLOT_ROWS * ((size_t)p.Ev + 2) * sizeof(float) + (size_t)p.Hkv * plan.rows * 2 * sizeof(int);
     }
     CHECK(plan.workspace_bytes >= need, "workspace");
     check_division((unsigned)plan.splits, (unsigned long long)plan.workgroups - 1, "workgroup id / splits");

@@ -287,7 +287,7 @@ def test_paged_plan_invariants():
     groups = 8 + 3500 // 128
     assert pl.row_blocks == 8 and pl.device_planned == 1 and pl.splits == 1
     assert pl.row_groups == groups + 32 and pl.workgroups == 8 * pl.row_groups
-    assert pl.workspace_bytes >= 8 * pl.row_groups * 128 * 130 * 4 + 3500 * 8
+    assert pl.workspace_bytes >= 8 * pl.row_groups * 128 * 130 * 4 + 8 * 3500 * 8
     pl = L.paged_plan(W=4, Hq=40, Hkv=8, Ev=128, block_size=16, max_blocks=783, num_cus=256, total_q=105)
     assert pl.row_blocks == 8 and pl.device_planned == 1 and pl.row_groups == 32 and pl.workgroups == 256
     # short tables: not more slots than there can be work for (four tiles per slot)
