@@ -223,12 +223,12 @@ typedef struct hw_paged_problem {
     const int32_t* cu_seqlens_q;   /* NULL selects the fixed-length operator */
     void* workspace;
     size_t workspace_bytes;
-    int32_t splits;            /* 0 = automatic; otherwise workgroups per (kv head, row group) */
-    int32_t row_blocks;        /* 0 = automatic; 1, 2 or 8 = 16-row MFMA blocks per workgroup (8: 128-row workgroups, 16-bit types,
-                                  max_blocks <= 8192; the automatic choice beyond 96 query rows per sequence and kv head --
-                                  for packed queries, whose lengths are device data, beyond 96 on average over the
-                                  sequences: a batch of one long and many one-token sequences stays on the 32-row kernel
-                                  unless the caller sets 8) */
+    int32_t splits;            /* 0 = automatic (packed queries in 128-row workgroups: decided on the device, see
+                                  hw_paged_plan.device_planned); otherwise workgroups per (kv head, row group) */
+    int32_t row_blocks;        /* 0 = automatic; 1, 2 or 8 = 16-row MFMA blocks per workgroup (8: workgroups of up to 128 rows
+                                  whose waves share every K/V tile, 16-bit types, max_blocks <= 8192; the automatic choice
+                                  beyond 16 query rows per sequence and kv head -- for packed queries, whose lengths are
+                                  device data, beyond 16 on average over the sequences) */
 } hw_paged_problem;
 
 typedef struct hw_paged_plan {
