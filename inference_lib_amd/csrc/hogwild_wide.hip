@@ -471,8 +471,8 @@ __device__ __forceinline__ void lds_transfer_flat(unsigned lds, unsigned long lo
 // all workgroups read, and a planning kernel in front of the launch cost 5.8 us plus the gap between two launches.
 // One thread per sequence and then per row group (at most PLAN_MAX_GROUPS of either; the host sends larger batches
 // down the unplanned path).  Every kv head has `pslots` workgroup slots.  A row group = up to 128 rows of one sequence;
-// its work is its sequence's tiles times the cost of a tile (a group of at most 64 rows multiplies one 16-row block per
-// wave instead of two: 0.6 against 0.8 us measured).  Every group takes one slot and a share of the others in
+// its work is its sequence's tiles times the cost of a tile (a group of at most 64 rows keeps one wave per SIMD busy
+// instead of two: 0.67 against 0.88 us per tile measured, 3 : 4).  Every group takes one slot and a share of the others in
 // proportion to its work (what the rounding leaves over goes to the groups with the most work per slot), four tiles per
 // slot at least; slots are numbered through the groups in order.  Returns what slot `item` does
 // (found = false: nothing), and -- for the workgroup that holds a group's first slot -- tells the merge kernel through
@@ -483,9 +483,11 @@ struct PlanSlot {
     int w, rg, qs, qe, split, ns;
     bool found;
 };
+template <int NTW>
 __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, int hkv, int GQ, int T, int tid) {
-    constexpr int NT = NTHREADS;
-    static_assert(NT == PLAN_MAX_GROUPS && WIDE_ROWS <= NT, "one thread per sequence, per row group, per row of a group");
+    constexpr int NT = PLAN_MAX_GROUPS;     // threads that take part (the others only meet the barriers)
+    static_assert(NTW >= NT && WIDE_ROWS <= NT, "one thread per sequence, per row group, per row of a group");
+    const bool act = tid < NT;
     int* sc_a = lds;                     // scan buffers
     int* sc_b = lds + NT;
     int* seq_qs = lds + 2 * NT;
@@ -493,8 +495,8 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
     int* seq_tiles = lds + 4 * NT;
     int* grp_w = lds + 5 * NT;
     int* grp_rg = lds + 6 * NT;
-    int* wave_part = lds + 7 * NT;       // [NT / 64]
-    int* shared = lds + 7 * NT + NT / 64;         // total of a scan; then the slot's entry (6 ints)
+    int* wave_part = lds + 7 * NT;       // [NTW / 64]
+    int* shared = lds + 7 * NT + NTW / 64;        // total of a scan; then the slot's entry (6 ints)
     const int lane = tid & 63, wv = tid >> 6;
     const int pslots = ph.nitems;
 
@@ -503,14 +505,14 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
     auto scan = [&](int v, int nact) {
         int* src = sc_a;
         int* dst = sc_b;
-        src[tid] = v;
+        if (act) src[tid] = v;
         __syncthreads();
         for (int off = 1; off < nact; off <<= 1) {
-            dst[tid] = src[tid] + (tid >= off ? src[tid - off] : 0);
+            if (act) dst[tid] = src[tid] + (tid >= off ? src[tid - off] : 0);
             __syncthreads();
             int* t = src; src = dst; dst = t;
         }
-        const int r = src[tid];
+        const int r = act ? src[tid] : 0;
         if (tid == nact - 1) shared[0] = r;
         __syncthreads();
         return r;
@@ -528,7 +530,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
         __syncthreads();
         int s = wave_part[0];
 #pragma unroll
-        for (int i = 1; i < NT / 64; ++i) s += wave_part[i];
+        for (int i = 1; i < NTW / 64; ++i) s += wave_part[i];
         return s;
     };
 
@@ -571,7 +573,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
     // what the rounding left over (fewer slots than groups) goes, one slot each, to the groups with the most work per slot
     const int left = pslots - block_total(n);
     const int load = (tid < G && n < most) ? __float_as_int((float)work * __builtin_amdgcn_rcpf((float)n)) : -1;   // (>= 0: ordered like the floats)
-    sc_a[tid] = load;
+    if (act) sc_a[tid] = load;
     __syncthreads();
     int ahead = 0;
     for (int g = 0; g < G; ++g) ahead += (sc_a[g] > load || (sc_a[g] == load && g < tid)) ? 1 : 0;
@@ -604,7 +606,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
         }
         if (item == 0) {
             const int covered = min(seq_qe[ph.W - 1] * GQ, ph.R);
-            for (int i = covered * 2 + tid; i < ph.R * 2; i += NT) row_tab[i] = 0;
+            for (int i = covered * 2 + tid; i < ph.R * 2; i += NTW) row_tab[i] = 0;
         }
     }
     return r;
@@ -617,13 +619,12 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
 // sequence's block table is copied into LDS once (up to PAGED_WIDE_MAX_BLOCKS entries; the launcher sends longer tables
 // to the narrow kernel).  Per tile every lane derives the cache rows it fetches from it; positions no row of the group
 // can see are redirected to the last visible one (no byte outside the visible part of the sequence is read; block ids
-// are clamped into the cache).
-template <class DT, int E, int EV, int NS>
-__global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHeader args) {
+// are clamped into the cache).  NW waves of 128 / NW rows each (see PAGED_WIDE_WAVES).
+template <class DT, int E, int EV, int NS, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeader args) {
 
     typedef Geo<DT, E, EV> G;
-    constexpr int NW = NWAVES;
-    constexpr int NT = NTHREADS;
+    constexpr int NT = NW * 64;
     constexpr int RB = WIDE_ROWS / 16 / NW;
     constexpr int WROWS = RB * 16;
     constexpr int TPR = NT / WIDE_ROWS;
@@ -685,7 +686,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     int w, rg, qs, qe, ns;
     size_t pbase;                           // row of the partial arrays that holds the workgroup's first row
     if (ph.flags & PH_PLANNED) {
-        const PlanSlot ps = plan_slot(ph, reinterpret_cast<int*>(ring), item, hkv, GQ, T, tid);   // (the ring is not in use yet)
+        const PlanSlot ps = plan_slot<NT>(ph, reinterpret_cast<int*>(ring), item, hkv, GQ, T, tid);   // (the ring is not in use yet)
         if (!ps.found) return;              // a slot the plan left empty; uniform over the workgroup
         w = __builtin_amdgcn_readfirstlane(ps.w);
         rg = __builtin_amdgcn_readfirstlane(ps.rg);
@@ -706,10 +707,6 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
     const int r0 = qs * GQ + rg * WIDE_ROWS;    // first row of the workgroup (global numbering: token * GQ + head in group)
     const int rend = qe * GQ;                   // end of the worker's rows
     if (r0 >= rend) return;                     // uniform over the workgroup
-    // A group of at most 64 rows (a short sequence, or the tail of a long one) is dealt 16 rows per wave instead of 32:
-    // every wave then has one 16-row block to multiply per tile instead of one wave two and the others none, and the
-    // workgroup's tile time, which the busiest wave sets, is that of one block.
-    const bool light = rend - r0 <= 16 * NW;    // uniform over the workgroup
     const int cap = ph.block_size * ph.max_blocks;
     const HW_GLOBAL int* btw = ph.block_table + (size_t)w * ph.max_blocks;
     const unsigned long long image = reinterpret_cast<unsigned long long>(k_wave ? ph.kcache : ph.vcache);
@@ -737,8 +734,9 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         for (int i = tid; i < nent; i += NT) bt_lds[i] = btw[i];
     }
 
-    // Everything from here on exists twice, for two and for one 16-row block per wave.  The branch is taken once per
-    // workgroup and the two copies share nothing but the values above, so each keeps the registers of its own tile loops.
+    // (The rest as a function of the 16-row blocks per wave, RBX.  With four waves of two blocks it used to be instantiated
+    // for one block as well, for row groups of at most 64 rows, behind one branch per workgroup: with the branch inside
+    // the fragment loop instead, the two copies shared their registers and the two-block tile loops ran 8 % slower.)
     auto run = [&](auto rbx) {
         constexpr int RBX = decltype(rbx)::value;
         constexpr int wrows = 16 * RBX;             // rows per wave
@@ -896,8 +894,7 @@ __global__ __launch_bounds__(NTHREADS, 1) void paged_wide_kernel(const PagedHead
         }
         HW_MARK(5);
     };
-    if (light) run(std::integral_constant<int, 1>{});
-    else run(std::integral_constant<int, RB>{});
+    run(std::integral_constant<int, RB>{});
 }
 
 // Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
@@ -928,11 +925,20 @@ hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStre
     }
 }
 
+// Waves per workgroup of the paged 128-row kernel: eight, two per SIMD, each with one 16-row block (so a row group of at
+// most 64 rows keeps half of them busy and one of at most 16 rows a single one).  Against four waves of two blocks --
+// where groups of at most 64 rows ran one block per wave, the same arithmetic per wave as here -- measured on four
+// 12 528-token sequences with 1/8/32/64, 1/1/1/64, 16 x 4 and 64 x 4 query tokens: 63.0 / 52.3 / 42.8 / 112.9 us against
+// 65.5 / 56.1 / 45.2 / 118.2 us; 7 x 4 and 12 x 4 tokens equal, 25 x 4 tokens 49.8 against 49.0 us.  (The fragment kernel
+// above stays with four: its tile loop runs at the pace of the tile stream either way.)
+constexpr int PAGED_WIDE_WAVES = 8;
+
 template <class DT>
 static hipError_t launch_paged_wide_dt(const PagedHeader& ph, int E, hipStream_t stream) {
     constexpr int NS = 5;      // ring slots: 5, 6 and 7 measure the same (a wave waits 4 ns per tile for its own transfers)
-    if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS>), dim3(ph.nwg), dim3(NTHREADS), 0, stream, ph);
-    else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS>), dim3(ph.nwg), dim3(NTHREADS), 0, stream, ph);
+    constexpr int NW = PAGED_WIDE_WAVES;
+    if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS, NW>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
+    else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS, NW>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
     return hipGetLastError();
 }
 

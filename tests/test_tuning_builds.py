@@ -29,7 +29,7 @@ def test_tuning_switches_still_compile(tmp_path, unit, flags):
 
 def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp_path):
     """The 128-row kernels issue their global->LDS tile transfers from inline assembly and count them by hand
-    (s_waitcnt vmcnt(12) or vmcnt(6): three tiles of four or two transfers may stay in flight).  The compiler does not know of them, and
+    (s_waitcnt vmcnt(12) ... vmcnt(3): three tiles of four to one transfers per wave may stay in flight).  The compiler does not know of them, and
     every wait it inserts itself for one of ITS loads inside a tile loop -- vmcnt(0), vmcnt(1): it counts only the loads
     it knows -- also waits for the look-ahead tiles and empties the pipeline at every tile; it has done so when a load's
     only use sat under a condition in front of the loop and the wait was left to the next touch of the register.  Checked
@@ -54,7 +54,10 @@ def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp
         for label, block in zip(parts[1::2], parts[2::2]):
             if "Depth=2" not in block:
                 continue                                   # not inside a tile loop (the loop over fragments / segments is depth 1)
-            ahead = 6 if "ELi64ELi64" in name else 12      # three tiles of two (head dimension 64) or four transfers per wave
+            # three tiles of (K + V bytes of a tile) / 1 KB / waves transfers per wave: head dimension and wave count from the name
+            m = re.search(r"ELi(\d+)ELi\d+ELi5E(?:Lb[01]E)?Li(\d+)E", name)
+            assert m, name
+            ahead = 3 * int(m.group(1)) // (8 * int(m.group(2)))
             for m in re.finditer(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", block):
                 checked += 1
                 assert int(m.group(1)) >= ahead, f"{name} {label}: {m.group(0)} inside a tile loop"
