@@ -193,6 +193,16 @@ def test_varlen_split_decided_on_the_device():
     check(c)
 
 
+def test_varlen_mixed_1_8_32_64_query_tokens():
+    """The shape of the packed-query benchmark at a size the oracle finishes: four sequences with 1 / 8 / 32 / 64 query
+    tokens at the QwQ-32B head shape (5 / 40 / 160 / 320 rows per kv head: row groups of 5, 40, 128 + 32 and 128 + 128 + 64
+    rows), planned on the device, against the oracle; and the launches with a fixed split agree with the same oracle."""
+    c = build_paged("bf16", 1, 4, 40, 8, 128, 16, 100, seq_lens=[1500, 1100, 1300, 1600], q_lens=[1, 8, 32, 64], seed=61)
+    check(c)
+    check(c, row_blocks=8, splits=3)
+    check(c, row_blocks=2)
+
+
 def test_varlen_tokens_behind_the_last_sequence_give_zeros():
     """total_q may exceed cu_seqlens_q[-1]: the tokens behind the last sequence belong to none.  The device-planned launch
     gives them zeros (lse -inf); the other launches leave them unspecified, like the reference, but must get the tokens of
