@@ -28,17 +28,18 @@
 
 namespace hw {
 
-// Phase timestamps of the 128-row kernels for tuning; compiled in only with -DHW_CLOCKS (never in the shipped library).
+// Phase timestamps of the 128-row kernels for tuning (the first four waves of a workgroup); compiled in only with
+// -DHW_CLOCKS (never in the shipped library).
 #ifdef HW_CLOCKS
 __device__ unsigned long long hw_wide_clock_buf[1024 * 4 * 16];
 #define HW_MARK(i)                                                                                  \
     do {                                                                                            \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
+        if ((threadIdx.x & 63) == 0 && threadIdx.x < 256 && blockIdx.x < 1024)                                        \
             hw_wide_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (i)] = wall_clock64();    \
     } while (0)
 #define HW_NOTE(i, v)                                                                               \
     do {                                                                                            \
-        if ((threadIdx.x & 63) == 0 && blockIdx.x < 1024)                                           \
+        if ((threadIdx.x & 63) == 0 && threadIdx.x < 256 && blockIdx.x < 1024)                                        \
             hw_wide_clock_buf[(blockIdx.x * 4 + (threadIdx.x >> 6)) * 16 + (i)] = (unsigned long long)(v); \
     } while (0)
 #else
@@ -483,6 +484,10 @@ struct PlanSlot {
     int w, rg, qs, qe, split, ns;
     bool found;
 };
+#ifndef HW_PLAN_W_HEAVY
+#define HW_PLAN_W_HEAVY 4
+#define HW_PLAN_W_LIGHT 3
+#endif
 template <int NTW>
 __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, int hkv, int GQ, int T, int tid) {
     constexpr int NT = PLAN_MAX_GROUPS;     // threads that take part (the others only meet the barriers)
@@ -562,7 +567,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
         gw = grp_w[tid];
         grg = grp_rg[tid];
         rows = min((seq_qe[gw] - seq_qs[gw]) * GQ - grg * WIDE_ROWS, WIDE_ROWS);
-        work = seq_tiles[gw] * (rows > WIDE_ROWS / 2 ? 4 : 3);
+        work = seq_tiles[gw] * (rows > WIDE_ROWS / 2 ? HW_PLAN_W_HEAVY : HW_PLAN_W_LIGHT);
         most = max(1, seq_tiles[gw] / 4);
     }
     // One slot each, and the other pslots - G in proportion to the work (rounded down, so they fit; the quotient in
@@ -619,32 +624,44 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
 // sequence's block table is copied into LDS once (up to PAGED_WIDE_MAX_BLOCKS entries; the launcher sends longer tables
 // to the narrow kernel).  Per tile every lane derives the cache rows it fetches from it; positions no row of the group
 // can see are redirected to the last visible one (no byte outside the visible part of the sequence is read; block ids
-// are clamped into the cache).  NW waves of 128 / NW rows each (see PAGED_WIDE_WAVES).
-template <class DT, int E, int EV, int NS, int NW>
+// are clamped into the cache).  NW waves: NW / PAR of them differ in their rows, and the PAR waves that share their rows
+// take the tiles of a step in turn and add up their partial sums at the end (see PAGED_WIDE_WAVES).
+template <class DT, int E, int EV, int NS, int NW, int PAR>
 __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeader args) {
 
     typedef Geo<DT, E, EV> G;
     constexpr int NT = NW * 64;
-    constexpr int RB = WIDE_ROWS / 16 / NW;
-    constexpr int WROWS = RB * 16;
+    constexpr int NRW = NW / PAR;                // waves that differ in their rows; PAR waves share the rows and alternate on the tiles
+    constexpr int RB = WIDE_ROWS / 16 / NRW;     // 16-row blocks per wave when the row group has more than 64 rows
     constexpr int TPR = NT / WIDE_ROWS;
-    constexpr int D = NS - 2;
+    constexpr int NSTEP = NS / PAR;              // ring slots in steps of PAR tiles (one barrier per step)
+    constexpr int DP = NSTEP - 1;                // steps requested ahead
     constexpr int KBYTES = G::KSTAGE;
     constexpr int VBYTES = TILE * G::VROW;
     constexpr int TPW = (KBYTES + VBYTES) / 1024 / NW;
+    constexpr int TPS = PAR * TPW;               // transfers a wave issues per step
     constexpr int SLOT = KBYTES + VBYTES;
     constexpr int RPL = 64 / G::CPR;             // tile rows one transfer covers
-    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && D >= 1 && NS >= 3 && G::KROW == G::VROW,
+    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && NS % PAR == 0 && DP >= 2 && G::KROW == G::VROW &&
+                      NW % PAR == 0 && (PAR == 1 || PAR == 2) && RB >= 1,
                   "16-bit types; a wave's transfers belong to one image");
 
-    __shared__ __attribute__((aligned(16))) char q_lds[WIDE_ROWS * G::QSTR];
+    // The rotated queries are needed in LDS only until every wave holds its rows as MFMA operands: they lie behind the
+    // ring slots that the first DP steps are requested into, in slots that are first requested into after the first
+    // barrier of the tile loop.
+    constexpr int QOFF = DP * PAR * SLOT;
+    constexpr int QBYTES = WIDE_ROWS * G::QSTR;
+    constexpr int RING_BYTES = NS * SLOT > QOFF + QBYTES ? NS * SLOT : QOFF + QBYTES;
     __shared__ int lim_lds[WIDE_ROWS];
     __shared__ int bt_lds[PAGED_WIDE_MAX_BLOCKS];
-    __shared__ __attribute__((aligned(16))) char ring[NS * SLOT];
+    __shared__ __attribute__((aligned(256))) char ring[RING_BYTES];
+    char* const q_lds = ring + QOFF;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rw = wv % NRW;                     // which rows
+    const int par = wv / NRW;                    // which tiles of a step
     const int n = lane & 15;
     const int q = lane >> 4;
 
@@ -734,13 +751,13 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
         for (int i = tid; i < nent; i += NT) bt_lds[i] = btw[i];
     }
 
-    // (The rest as a function of the 16-row blocks per wave, RBX.  With four waves of two blocks it used to be instantiated
-    // for one block as well, for row groups of at most 64 rows, behind one branch per workgroup: with the branch inside
-    // the fragment loop instead, the two copies shared their registers and the two-block tile loops ran 8 % slower.)
+    // (The rest as a function of the 16-row blocks per wave, RBX: two for row groups of more than 64 rows, one for the
+    // others, behind one branch per workgroup.  With the branch inside the fragment loop instead, the two copies shared
+    // their registers and the two-block tile loops ran 8 % slower.)
     auto run = [&](auto rbx) {
         constexpr int RBX = decltype(rbx)::value;
         constexpr int wrows = 16 * RBX;             // rows per wave
-        const int w0 = r0 + wv * wrows;             // first row of this wave
+        const int w0 = r0 + rw * wrows;             // first row of this wave
         WaveState<RBX, G::NOC> st;
 #pragma unroll
         for (int rb = 0; rb < RBX; ++rb) {
@@ -752,20 +769,25 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
         st.fresh = true;
 
         for (int f = 0; f < ph.F; ++f) {
+            // (the thread index as the compiler cannot see through it: what the prologue derives from it -- rows, addresses of
+            // the queries -- is then formed here, per fragment, instead of once in front of the loop, from where it would stay
+            // in registers across the tile loops, which have none to spare)
+            int tidf = tid;
+            asm volatile("" : "+v"(tidf));
             QueryRotation<DT, E, WIDE_ROWS, G::QSTR, true, NT> qrot;
-            qrot.load(a, f, hkv, r0, GQ, tid);
-            const int lm = ph.loc[(size_t)f * T + fast_div(min(r0 + tid / TPR, rend - 1), ph.magic_gq)];
+            qrot.load(a, f, hkv, r0, GQ, tidf);
+            const int lm = ph.loc[(size_t)f * T + fast_div(min(r0 + tidf / TPR, rend - 1), ph.magic_gq)];
             const int flen = ph.frag_len[ph.cu_q != nullptr ? f * ph.W + w : f];
 
             __syncthreads();   // the previous fragment's readers are done with q_lds / lim_lds / the ring
             if (f == 0) HW_MARK(7);
-            qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tid);
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tidf);
             // (computed by every thread and pinned there: the compiler waits for a load where its result is first used, and a
             // use under the condition below leaves the wait to whatever next touches the registers -- inside the tile loops,
             // where a wait for "all loads" also waits for the look-ahead transfers it does not know of)
-            int limv = (r0 + tid / TPR < rend) ? max(0, min(min(flen, cap), lm < cap ? lm + 1 : cap)) : 0x7fffffff;
+            int limv = (r0 + tidf / TPR < rend) ? max(0, min(min(flen, cap), lm < cap ? lm + 1 : cap)) : 0x7fffffff;
             asm volatile("" : "+v"(limv));
-            if (tid % TPR == 0) lim_lds[tid / TPR] = limv;
+            if (tidf % TPR == 0) lim_lds[tidf / TPR] = limv;
             __syncthreads();
             if (f == 0) HW_MARK(1);
 
@@ -775,12 +797,12 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
                 for (int rb = 0; rb < RBX; ++rb)
 #pragma unroll
                     for (int j = 0; j < G::KJ; ++j)
-                        qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * wrows + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+                        qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (rw * wrows + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
                 int lim[RBX];
                 int maxlim = 0, minlim = 0x7fffffff;
 #pragma unroll
                 for (int rb = 0; rb < RBX; ++rb) {
-                    lim[rb] = lim_lds[wv * wrows + rb * 16 + n];
+                    lim[rb] = lim_lds[rw * wrows + rb * 16 + n];
                     const bool pad = w0 + rb * 16 + n >= rend;
                     maxlim = max(maxlim, pad ? 0 : lim[rb]);
                     minlim = min(minlim, lim[rb]);
@@ -788,7 +810,7 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
                 maxlim = __builtin_amdgcn_readfirstlane(row_max16(maxlim));
                 minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
                 // what the WORKGROUP can see decides which positions are fetched and where its tile loop ends (every wave must
-                // take part in every tile's barrier); what the wave can see decides which tiles it multiplies
+                // take part in every step's barrier); what the wave can see decides which tiles it multiplies
                 int wgmax = 0;
 #pragma unroll
                 for (int i = 0; i < WIDE_ROWS / 64; ++i) {
@@ -799,64 +821,76 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
                 for (int off = 1; off < 64; off <<= 1) wgmax = max(wgmax, __shfl_xor(wgmax, off, 64));
                 wgmax = __builtin_amdgcn_readfirstlane(wgmax);
 
-                // Source addresses of this wave's share of tile t (TPW transfers): every lane looks up the block of the row it
-                // fetches in each transfer.  A position beyond what the workgroup can see is replaced by the last visible one, so a
-                // tile that does not exist costs the same number of transfers and no new memory traffic to speak of, and no byte
-                // outside the visible part of the sequence is read.
-                auto addresses = [&](unsigned long long* src, int t) {
+                // Source addresses of this wave's share of the PAR tiles of the step that starts at tile tb (TPS transfers):
+                // every lane looks up the block of the row it fetches in each transfer.  A position beyond what the workgroup
+                // can see is replaced by the last visible one, so a tile that does not exist costs the same number of
+                // transfers and no new memory traffic to speak of, and no byte outside the visible part of the sequence is
+                // read.
+                auto addresses = [&](unsigned long long* src, int tb) {
 #pragma unroll
-                    for (int j = 0; j < TPW; ++j) {
-                        const int tok = min(t * TILE + trow[j], wgmax - 1);
-                        const int bi = fast_div(tok, ph.magic_bs);
-                        const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
-                        const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
-                        src[j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
-                    }
+                    for (int pp = 0; pp < PAR; ++pp)
+#pragma unroll
+                        for (int j = 0; j < TPW; ++j) {
+                            const int tok = min((tb + pp * ns) * TILE + trow[j], wgmax - 1);
+                            const int bi = fast_div(tok, ph.magic_bs);
+                            const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
+                            const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
+                            src[pp * TPW + j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
+                        }
                 };
-                auto request = [&](int sl, const unsigned long long* src) {
+                auto request = [&](int step_slot, const unsigned long long* src) {
 #pragma unroll
-                    for (int j = 0; j < TPW; ++j) lds_transfer_flat(__builtin_amdgcn_readfirstlane(my_image + sl * SLOT + j * 1024), src[j]);
+                    for (int pp = 0; pp < PAR; ++pp)
+#pragma unroll
+                        for (int j = 0; j < TPW; ++j)
+                            lds_transfer_flat(__builtin_amdgcn_readfirstlane(my_image + (step_slot * PAR + pp) * SLOT + j * 1024), src[pp * TPW + j]);
                 };
 
                 if (wgmax > 0) {   // uniform over the workgroup
-                    // tiles of this workgroup: split, split + nsplit, ...  The addresses of a request are formed one tile earlier
-                    // (after the barrier, next to the arithmetic): the request at the top of a tile is then four transfers and
-                    // nothing else, and no wave reaches the barrier late because it was still looking up blocks.
-                    unsigned long long src[TPW];
+                    // Tiles of this workgroup: split, split + ns, ...; a step is PAR of them, one for each of the waves that
+                    // share their rows, behind one barrier.  The first DP steps are requested here; every later one right
+                    // behind the barrier that frees its slots (all waves have left the step before), with addresses formed a
+                    // step earlier, next to the arithmetic: a request is then TPS transfers and nothing else.
+                    const int tstep = PAR * ns;
+                    int first_tile = __builtin_amdgcn_readfirstlane(split);   // (opaque, like tidf: the positions of the first steps are formed here)
+                    asm volatile("" : "+s"(first_tile));
+                    unsigned long long src[TPS];
 #pragma unroll
-                    for (int i = 0; i < D; ++i) {
-                        addresses(src, split + i * ns);
+                    for (int i = 0; i < DP; ++i) {
+                        addresses(src, first_tile + i * tstep);
                         request(i, src);
                     }
-                    addresses(src, split + D * ns);
+                    addresses(src, first_tile + DP * tstep);
+                    // (the operands and bounds read out of LDS above have arrived before any wave passes the first barrier and
+                    // requests into the slots the queries lie in)
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                     // two loops with one instantiation of the tile arithmetic each (see attention_wide_kernel)
-                    int sl = 0;
-                    int t = split;
-                    auto arrive = [&]() {                         // request tile t + D * ns, wait for tile t, form the next addresses
-                        int rs = sl + D;
-                        if (rs >= NS) rs -= NS;
-                        request(rs, src);
-                        // this wave's transfers of tile t have landed (the D requests issued since may stay in flight: loads
-                        // complete in order), then every wave's: a plain barrier, no fence that would wait for the look-ahead
-                        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
-                        addresses(src, t + (D + 1) * ns);
+                    int sl = 0;                                   // step slot of the current step
+                    int tb = first_tile;                          // its first tile
+                    auto arrive = [&]() {
+                        // this wave's transfers of the step have landed (the DP - 1 steps requested since may stay in flight:
+                        // loads complete in order), then every wave's: a plain barrier, no fence that would wait for the
+                        // look-ahead.  Behind it the slots of the step before are free: request step + DP into them.
+                        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DP - 1) * TPS) : "memory");
+                        request(sl == 0 ? NSTEP - 1 : sl - 1, src);
+                        addresses(src, tb + (DP + 1) * tstep);
                     };
                     const int tfast = maxlim > 0 ? min(minlim, wgmax) / TILE : 0;   // tiles below it are seen completely by every row of the wave
 #pragma unroll 1
-                    for (; t < tfast; t += ns) {
+                    for (; tb + par * ns < tfast; tb += tstep) {
                         arrive();
-                        const char* slot = ring + sl * SLOT;
-                        compute_tile<DT, E, EV, RBX, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
-                        sl = sl + 1 == NS ? 0 : sl + 1;
+                        const char* slot = ring + (sl * PAR + par) * SLOT;
+                        compute_tile<DT, E, EV, RBX, false, true, false, true, (RBX > 1)>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                        sl = sl + 1 == NSTEP ? 0 : sl + 1;
                     }
 #pragma unroll 1
-                    for (; t * TILE < wgmax; t += ns) {           // uniform over the workgroup: every wave leaves at the same tile
+                    for (; tb * TILE < wgmax; tb += tstep) {      // uniform over the workgroup: every wave leaves at the same step
                         arrive();
-                        if (t * TILE < maxlim) {
-                            const char* slot = ring + sl * SLOT;
-                            compute_tile<DT, E, EV, RBX, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                        if ((tb + par * ns) * TILE < maxlim) {
+                            const char* slot = ring + (sl * PAR + par) * SLOT;
+                            compute_tile<DT, E, EV, RBX, true, true, false, true, (RBX > 1)>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                         }
-                        sl = sl + 1 == NS ? 0 : sl + 1;
+                        sl = sl + 1 == NSTEP ? 0 : sl + 1;
                     }
                     // the requests behind the last tile must have landed before the ring is used again
                     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -864,16 +898,48 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
             }
         }
 
-        // ---- every wave stores the partial of its own rows, 16-row blocks staged through the ring (see attention_wide_kernel) ----
+        // ---- The PAR waves that share their rows hold a partial sum each: block rb of the rows goes to wave rb % PAR of
+        // them through LDS (the ring, which no tile needs any more), lane for lane in the accumulator layout, and is
+        // combined there.  Every wave then stores the blocks it owns, staged through LDS once more so that they leave as
+        // whole rows (see attention_wide_kernel). ----
         {
             constexpr int OSTR = EV + 4;
-            static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+            constexpr int REGION = 16 * OSTR;                     // floats per wave: a staged 16-row block, or a block in accumulator layout
+            static_assert(G::NOC * 64 * 4 <= REGION && (NW * REGION + NW * 64 * 2) * 4 <= RING_BYTES, "the blocks of all waves fit into the ring");
             HW_MARK(3);
             __syncthreads();
-            float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
+            float* const regions = reinterpret_cast<float*>(ring);
+            float* const mls = regions + NW * REGION;
+            if constexpr (PAR > 1) {
+#pragma unroll
+                for (int rb = 0; rb < RBX; ++rb) {
+                    const int owner = rw + (rb % PAR) * NRW;
+                    if (owner != wv) {
+#pragma unroll
+                        for (int c = 0; c < G::NOC; ++c) *reinterpret_cast<f32x4*>(regions + owner * REGION + (c * 64 + lane) * 4) = st.o[rb][c];
+                        *reinterpret_cast<f32x2*>(mls + (owner * 64 + lane) * 2) = f32x2{st.m[rb], st.l[rb]};
+                    }
+                }
+                __syncthreads();
+            }
+            float* stage = regions + wv * REGION;
             {
 #pragma unroll
                 for (int rb = 0; rb < RBX; ++rb) {
+                    if (rw + (rb % PAR) * NRW != wv) continue;    // uniform over the wave
+                    if constexpr (PAR > 1) {
+                        const f32x2 oml = *reinterpret_cast<const f32x2*>(mls + (wv * 64 + lane) * 2);
+                        const float mnew = fmaxf(st.m[rb], oml.x);
+                        const float mine = exp2f(st.m[rb] - mnew), theirs = exp2f(oml.x - mnew);
+#pragma unroll
+                        for (int c = 0; c < G::NOC; ++c) {
+                            const f32x4 o2 = *reinterpret_cast<const f32x4*>(stage + (c * 64 + lane) * 4);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) st.o[rb][c][i] = st.o[rb][c][i] * mine + o2[i] * theirs;
+                        }
+                        st.l[rb] = st.l[rb] * mine + oml.y * theirs;
+                        st.m[rb] = mnew;
+                    }
                     const float lsum = quarter_sum(st.l[rb]);
                     const int row0 = w0 + rb * 16;
                     const size_t prow0 = pbase + (size_t)(row0 - r0);
@@ -894,7 +960,8 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
         }
         HW_MARK(5);
     };
-    run(std::integral_constant<int, RB>{});
+    if (RB > 1 && rend - r0 <= WIDE_ROWS / 2) run(std::integral_constant<int, RB / 2>{});
+    else run(std::integral_constant<int, RB>{});
 }
 
 // Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
@@ -925,20 +992,33 @@ hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStre
     }
 }
 
-// Waves per workgroup of the paged 128-row kernel: eight, two per SIMD, each with one 16-row block (so a row group of at
-// most 64 rows keeps half of them busy and one of at most 16 rows a single one).  Against four waves of two blocks --
-// where groups of at most 64 rows ran one block per wave, the same arithmetic per wave as here -- measured on four
-// 12 528-token sequences with 1/8/32/64, 1/1/1/64, 16 x 4 and 64 x 4 query tokens: 63.0 / 52.3 / 42.8 / 112.9 us against
-// 65.5 / 56.1 / 45.2 / 118.2 us; 7 x 4 and 12 x 4 tokens equal, 25 x 4 tokens 49.8 against 49.0 us.  (The fragment kernel
-// above stays with four: its tile loop runs at the pace of the tile stream either way.)
+// Waves per workgroup of the paged 128-row kernel: eight, two per SIMD.  The two waves of a SIMD share their rows (32
+// rows = two 16-row blocks for a row group of more than 64 rows, else one block) and take every other tile: a step of the
+// tile loop is two tiles behind one barrier, one for each of them.  So each wave reads half of the tiles out of LDS, and
+// the arithmetic of one runs beside the waits of the other.  Measured on four 12 528-token sequences with 1/8/32/64,
+// 1/1/1/64, 16 x 4, 64 x 4, 25 x 4 and 12 x 4 query tokens, against eight waves of 16 rows that all take every tile (which
+// doubles what is read out of LDS per tile and row): 57.9 / 48.2 / 42.3 / 110.0 / 47.3 / 40.1 us against 64.7 / 52.4 / 43.4 /
+// 116.4 / 50.6 / 39.2 us; that form had in turn been 4 % faster than four waves of 32 rows on every tile (one per SIMD).
+// Ring of six 16 KB slots = three steps: one being multiplied, two in flight.  The two-block instantiation fits the 256
+// registers of a wave exactly (see LEAN in compute_tile); a spill there costs more than the registers it frees, because
+// the compiler's wait for the reload also waits for the tile transfers in flight.
+#ifndef HW_PAGED_WIDE_PAR
+#define HW_PAGED_WIDE_PAR 2
+#endif
+#ifndef HW_PAGED_WIDE_SLOTS
+#define HW_PAGED_WIDE_SLOTS 6
+#endif
 constexpr int PAGED_WIDE_WAVES = 8;
+constexpr int PAGED_WIDE_PAR = HW_PAGED_WIDE_PAR;
+constexpr int PAGED_WIDE_SLOTS = HW_PAGED_WIDE_SLOTS;
 
 template <class DT>
 static hipError_t launch_paged_wide_dt(const PagedHeader& ph, int E, hipStream_t stream) {
-    constexpr int NS = 5;      // ring slots: 5, 6 and 7 measure the same (a wave waits 4 ns per tile for its own transfers)
+    constexpr int NS = PAGED_WIDE_SLOTS;
     constexpr int NW = PAGED_WIDE_WAVES;
-    if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS, NW>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
-    else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS, NW>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
+    constexpr int PAR = PAGED_WIDE_PAR;
+    if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS, NW, PAR>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
+    else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS, NW, PAR>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
     return hipGetLastError();
 }
 

@@ -28,12 +28,13 @@ def test_tuning_switches_still_compile(tmp_path, unit, flags):
 
 
 def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp_path):
-    """The 128-row kernels issue their global->LDS tile transfers from inline assembly and count them by hand
-    (s_waitcnt vmcnt(12) ... vmcnt(3): three tiles of four to one transfers per wave may stay in flight).  The compiler does not know of them, and
-    every wait it inserts itself for one of ITS loads inside a tile loop -- vmcnt(0), vmcnt(1): it counts only the loads
-    it knows -- also waits for the look-ahead tiles and empties the pipeline at every tile; it has done so when a load's
-    only use sat under a condition in front of the loop and the wait was left to the next touch of the register.  Checked
-    in the generated code: inside the innermost loops of both kernels no wait for vector memory below the look-ahead."""
+    """The 128-row kernels issue their global->LDS tile transfers from inline assembly and count them by hand (s_waitcnt
+    vmcnt(n) in front of each barrier, n = the transfers of the look-ahead that may stay in flight).  The compiler does not
+    know of them, and every wait it inserts itself for one of ITS loads inside a tile loop -- vmcnt(0), vmcnt(1): it counts
+    only the loads it knows -- also waits for the look-ahead tiles and empties the pipeline at every tile; it has done so
+    when a load's only use sat under a condition in front of the loop and the wait was left to the next touch of the
+    register, and when a register spilled in front of the loop was reloaded there.  Checked in the generated code: inside
+    the innermost loops of both kernels no wait for vector memory below the look-ahead, and no scratch memory at all."""
     if shutil.which(HIPCC) is None and not os.path.exists(HIPCC):
         pytest.skip("no hipcc")
     import re
@@ -49,15 +50,29 @@ def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp
     checked = 0
     for name in kernels:
         body = text[text.index(name + ":"):]
-        body = body[:body.index("; -- End function")]
+        end = body.index("; -- End function")
+        # (a register spilled anywhere is reloaded with a wait for "all loads", which in front of the tile loops also waits
+        # for the first tiles' transfers)
+        scratch = re.search(r"; ScratchSize: (\d+)", body[end:end + 4000])
+        assert scratch and int(scratch.group(1)) == 0, f"{name}: {scratch and scratch.group(0)}"
+        body = body[:end]
         parts = re.split(r"\n(\.LBB\d+_\d+):", body)
         for label, block in zip(parts[1::2], parts[2::2]):
             if "Depth=2" not in block:
                 continue                                   # not inside a tile loop (the loop over fragments / segments is depth 1)
-            # three tiles of (K + V bytes of a tile) / 1 KB / waves transfers per wave: head dimension and wave count from the name
-            m = re.search(r"ELi(\d+)ELi\d+ELi5E(?:Lb[01]E)?Li(\d+)E", name)
-            assert m, name
-            ahead = 3 * int(m.group(1)) // (8 * int(m.group(2)))
+            # a wave issues E / (8 * waves) transfers per tile (K + V bytes of a tile / 1 KB / waves); head dimension, ring
+            # slots, waves and the tiles per step from the name
+            m = re.search(r"attention_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELb[01]ELi(\d+)E", name)
+            if m:       # three tiles requested ahead of the one that is waited for
+                e, ns, nw = (int(x) for x in m.groups())
+                ahead = (ns - 2) * e // (8 * nw)
+            else:       # steps of `par` tiles, requested behind the barrier: one step stays in flight
+                m = re.search(r"paged_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELi(\d+)ELi(\d+)E", name)
+                assert m, name
+                e, ns, nw, par = (int(x) for x in m.groups())
+                ahead = (ns // par - 2) * par * e // (8 * nw)
+            assert ahead >= 1, name
+            assert "scratch_" not in block, f"{name} {label}: scratch memory inside a tile loop"
             for m in re.finditer(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", block):
                 checked += 1
                 assert int(m.group(1)) >= ahead, f"{name} {label}: {m.group(0)} inside a tile loop"
