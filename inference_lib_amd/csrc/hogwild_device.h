@@ -279,10 +279,6 @@ __device__ __forceinline__ u32x2 lds_read_tr16(const char* p) {
     const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(p));
     return __builtin_bit_cast(u32x2, r);
 }
-__device__ __forceinline__ u32x2 lds_read_tr16_at(unsigned lds_byte) {
-    const v4i16 r = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4i16*)(size_t)lds_byte);
-    return __builtin_bit_cast(u32x2, r);
-}
 // Per-lane byte offsets into a swizzled V image for output block c (16 elements) and the first 16 tokens of a tile (the
 // lane names row 4q + r, r = (lane / 4) % 4, piece lane % 4); add 16 * VROW for the second 16 tokens (same key).
 template <int VROW>
@@ -309,10 +305,7 @@ struct WaveState {
 // kernels whose waves share every tile, 16-bit types): the K operands are read first (LDS answers in order, and the
 // logits wait for K only), the V^T operands come straight out of the image (lds_read_tr16, per-lane offsets `voff` from
 // vtr_lane_offsets), and output block c then holds elements 16c .. 16c+15.  `t_in` is not used.
-// LEAN (with VLDS) = for a kernel whose tile loop has no registers to spare: the K operands are read one 16-token block
-// at a time, and the V^T reads form their addresses from voff[0] alone (the blocks of a lane differ in address bits
-// 5 .. 7 only, which the swizzle key and the block number share by XOR; `vimg` must then be aligned to 256 bytes).
-template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false, bool LEAN = false>
+template <class DT, int E, int EV, int RB, bool MASKED, bool QREG, bool VS = false, bool VLDS = false>
 __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, const char* q_lds, const u32x4* qreg, const int (&lim)[RB],
                                              WaveState<RB, Geo<DT, E, EV>::NOC>& st, int t0, int n, int q, float sc, const char* kstage,
                                              const char* vimg = nullptr, const unsigned* voff = nullptr) {
@@ -352,20 +345,6 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
                     for (int d = 0; d < 4; ++d) acc = Elem<DT>::dot(kk[d], qq[d], acc);
                 }
                 sacc[rb][idx >> 2][idx & 3] = acc;
-            }
-        }
-    } else if constexpr (VLDS && LEAN) {
-#pragma unroll
-        for (int tb = 0; tb < 2; ++tb) {
-            u32x4 kop[G::KJ];
-#pragma unroll
-            for (int j = 0; j < G::KJ; ++j) kop[j] = *reinterpret_cast<const u32x4*>(kstage + kstage_offset<G>(tb * 16 + n, 4 * j + q));
-#pragma unroll
-            for (int rb = 0; rb < RB; ++rb) {
-                f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int j = 0; j < G::KJ; ++j) acc = Elem<DT>::mfma(kop[j], qreg[rb * G::KJ + j], acc);
-                sacc[rb][tb] = acc;
             }
         }
     } else if constexpr (VLDS) {
@@ -414,23 +393,14 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
     // output products below then issue back to back.  (Read where they are used, one chunk's pair of reads at a time into
     // the same registers, every chunk waited for the LDS round trip in front of its two products: eight exposed round
     // trips per tile.)
-    // (LEAN: the first half of them here, the second half behind the exponentials, when the logits' registers are free.)
     [[maybe_unused]] u32x4 vops[VLDS ? G::NOC : 1];
-    constexpr int NV_EARLY = LEAN ? G::NOC / 2 : G::NOC;
-    [[maybe_unused]] auto read_vop = [&](int c) {
-        u32x2 a0, a1;
-        if constexpr (LEAN) {
-            const unsigned va = ((unsigned)(size_t)HW_LDS_PTR(vimg) + voff[0]) ^ (unsigned)(c << 5);
-            a0 = lds_read_tr16_at(va), a1 = lds_read_tr16_at(va + 16 * G::VROW);
-        } else {
-            const char* vp = vimg + voff[c];
-            a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
-        }
-        vops[c] = u32x4{a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
-    };
     if constexpr (VLDS) {
 #pragma unroll
-        for (int c = 0; c < NV_EARLY; ++c) read_vop(c);
+        for (int c = 0; c < G::NOC; ++c) {
+            const char* vp = vimg + voff[c];
+            const u32x2 a0 = lds_read_tr16(vp), a1 = lds_read_tr16(vp + 16 * G::VROW);
+            vops[c] = u32x4{a0.x, a0.y, a1.x, a1.y};     // tokens slot_token(q, 0..7) of element 16c + n
+        }
         __builtin_amdgcn_sched_barrier(0);
     }
     // Online softmax with a lazily updated reference: exponentials are taken against st.m, which only moves when
@@ -439,7 +409,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
     // registers.  p is at most 2^LAZY_LOG2, far inside the range of every storage type.
     constexpr float LAZY_LOG2 = 8.0f;
     float s[RB][8];
-    float mxs[RB];
+    float mxl[RB];     // maximum over this lane's eight tokens (a quarter of the tile)
     bool need = false;
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
@@ -450,15 +420,19 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             if constexpr (MASKED) s[rb][idx] = (t0 + slot_token(q, idx)) < lim[rb] ? s[rb][idx] : NEG_BIG;
             mx = fmaxf(mx, s[rb][idx]);
         }
-        mx = quarter_max(mx);
+        mxl[rb] = mx;
+        // A row's maximum exceeds the bound exactly when that of one of its four lanes does: the test needs no
+        // reduction across the lanes, which is left to the (rare) branch that moves the reference.
         // sc > 0: scaling commutes with the max; a row that sees nothing of a masked tile keeps NEG_BIG
-        mxs[rb] = MASKED ? (mx < -1.0e29f ? NEG_BIG : mx * sc) : mx * sc;
-        need = need || (mxs[rb] > st.m[rb] + LAZY_LOG2);
+        const float mine = MASKED ? (mx < -1.0e29f ? NEG_BIG : mx * sc) : mx * sc;
+        need = need || (mine > st.m[rb] + LAZY_LOG2);
     }
     if (__builtin_amdgcn_ballot_w64(need) != 0) {        // uniform over the wave
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-            const float mnew = mxs[rb] > st.m[rb] + LAZY_LOG2 ? mxs[rb] : st.m[rb];
+            const float mx = quarter_max(mxl[rb]);
+            const float mxs = MASKED ? (mx < -1.0e29f ? NEG_BIG : mx * sc) : mx * sc;
+            const float mnew = mxs > st.m[rb] + LAZY_LOG2 ? mxs : st.m[rb];
             const float alpha = fast_exp2(st.m[rb] - mnew);   // 1 for rows that keep their reference
             st.m[rb] = mnew;
             st.l[rb] *= alpha;
@@ -493,8 +467,6 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
             pp[rb].w = Elem<DT>::pack2(p[rb][6], p[rb][7]);
         }
         if constexpr (VLDS) {
-#pragma unroll
-            for (int c = NV_EARLY; c < G::NOC; ++c) read_vop(c);
 #pragma unroll
             for (int c = 0; c < G::NOC; ++c) {
                 const u32x4 vop = vops[c];

@@ -1,23 +1,25 @@
 // Hogwild! fragmented-KV attention for many query rows per kv head (several tokens per worker, many workers, wide GQA
 // groups): the shape where a decode step turns into a small prefill.  gfx950 (MI355X, CDNA4, wave64), 16-bit types.
 //
-// One workgroup = one kv head x one contiguous range of 32-token tiles x up to 128 query rows: each of the four
-// waves owns 32 rows (two 16-row MFMA blocks) and ALL four multiply against EVERY tile of the range.  A tile is brought
-// into LDS once per workgroup -- K and V by direct global->LDS transfers, the K image issued by the first half of the
-// waves and the V image by the second -- and read from there by all of them.  What bounds the narrow kernel on such shapes is the rate at which one CU can
-// take data in (about 16 B/clk through the vector memory path, whatever cache answers): with 32-row workgroups every
-// group of 32 rows streams the whole KV through its CU again, four times for 128 rows.  Here a CU takes every byte in
-// once and spreads it through LDS (each wave reads 16 KB per tile out of 128 B/clk of LDS bandwidth).
+// One workgroup = one kv head x one contiguous range of 32-token tiles x up to 128 query rows, eight waves: four groups
+// of 32 rows (two 16-row MFMA blocks), and the two waves of a group -- the two waves of one SIMD -- take every other
+// tile.  A tile is brought into LDS once per workgroup -- K and V by direct global->LDS transfers, every wave issuing its
+// share -- and read from there by the four waves whose turn it is.  What bounds the narrow kernel on such shapes is the
+// rate at which one CU can take data in (about 16 B/clk through the vector memory path, whatever cache answers): with
+// 32-row workgroups every group of 32 rows streams the whole KV through its CU again, four times for 128 rows.  Here a
+// CU takes every byte in once and spreads it through LDS (a wave reads 16 KB per tile it multiplies out of 128 B/clk of
+// LDS bandwidth; with one wave per SIMD taking every tile the arithmetic of a tile had nothing to run beside, with two
+// waves per SIMD that both take every tile the LDS reads double).
 //
-// The tiles rotate through a ring of NS LDS slots; D = NS - 2 tiles are requested ahead.  One barrier per tile: a wave
-// waits for its own transfers of tile t, all waves meet, tile t is complete in LDS; and since every wave has then left
-// tile t-1 behind, the slot of tile t-1 is free for the request issued next (tile t+D goes to slot (t+D) mod NS, which
-// is neither the slot being read nor one still in flight).  The transfers are issued from inline assembly and waited for
-// by hand (see lds_transfer).
-// Rows of different waves are different rows, so nothing is combined across waves at the end: every wave stores the
-// partial (unnormalised output, running max, sum) of its own 32 rows, and the merge kernel of the narrow path
-// (merge_kernel) finishes the job.
-
+// The tiles rotate through a ring of NS LDS slots in steps of PAR = 2 tiles, one for each wave of a group.  One barrier
+// per step: a wave waits for its own transfers of the step, all waves meet, the step is complete in LDS; and since every
+// wave has then left the step before behind, its slots are free for the request issued right behind the barrier (NS / PAR
+// - 1 steps are in flight or being multiplied).  The transfers are issued from inline assembly and waited for by hand
+// (see lds_transfer).
+// The two waves of a group add up their partial sums through LDS at the end (each takes one 16-row block of the 32
+// rows); rows of different groups are different rows.  Every wave then stores the partial (unnormalised output, running
+// max, sum) of its block, and the merge kernel of the narrow path (merge_kernel) finishes the job.
+//
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -111,8 +113,8 @@ struct WideRotation {
     u32x4 xa[NIT], xb[NIT];
     f32x4 tab[NCS];
 
-    // global loads: the queries of this thread's chunk pairs and its share of the table rows ws_lo .. ws_lo + nws - 1
-    __device__ __forceinline__ void load(const DevHeader& a, int f, int hkv, int r0, int GQ, int tid, int ws_lo, int nws) {
+    // global loads: the queries of this thread's chunk pairs (the same for every fragment) ...
+    __device__ __forceinline__ void load_queries(const DevHeader& a, int hkv, int r0, int GQ, int tid) {
 #pragma unroll
         for (int it = 0; it < NIT; ++it) {
             const int item = tid + it * NT;
@@ -123,6 +125,9 @@ struct WideRotation {
             xa[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + slot * 16);
             xb[it] = *reinterpret_cast<const HW_GLOBAL u32x4*>(qp + (slot + IPR) * 16);
         }
+    }
+    // ... and its share of fragment f's table rows ws_lo .. ws_lo + nws - 1
+    __device__ __forceinline__ void load_tables(const DevHeader& a, int f, int tid, int ws_lo, int nws) {
 #pragma unroll
         for (int k = 0; k < NCS; ++k) {
             const int item = tid + k * NT;
@@ -175,19 +180,23 @@ struct WideRotation {
     }
 };
 
-template <class DT, int E, int EV, int NS, bool PRE, int NW>
+template <class DT, int E, int EV, int NS, bool PRE, int NW, int PAR>
 __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const KernelArgs args) {
     typedef Geo<DT, E, EV> G;
     constexpr int NT = NW * 64;                 // threads per workgroup
-    constexpr int RB = WIDE_ROWS / 16 / NW;     // 16-row blocks per wave
+    constexpr int NRW = NW / PAR;               // waves that differ in their rows; PAR waves share the rows and alternate on the tiles
+    constexpr int RB = WIDE_ROWS / 16 / NRW;    // 16-row blocks per wave
     constexpr int WROWS = RB * 16;              // rows per wave
     constexpr int TPR = NT / WIDE_ROWS;         // threads per row where a row is handled by a group of threads
-    constexpr int D = NS - 2;                   // tiles requested ahead
+    constexpr int NSTEP = NS / PAR;             // ring slots in steps of PAR tiles (one barrier per step)
+    constexpr int DP = NSTEP - 1;               // steps requested ahead
     constexpr int KBYTES = G::KSTAGE;           // K image of a tile in LDS
     constexpr int VBYTES = TILE * G::VROW;      // V image
     constexpr int TPW = (KBYTES + VBYTES) / 1024 / NW;   // 1 KB transfers each wave issues per tile
+    constexpr int TPS = PAR * TPW;              // ... per step
     constexpr int SLOT = KBYTES + VBYTES;
-    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && D >= 1 && RB >= 1 && NS >= 3,
+    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && NS % PAR == 0 && DP >= 1 && RB >= 1 &&
+                      NW % PAR == 0 && (PAR == 1 || PAR == 2),
                   "16-bit types; a wave's transfers belong to one image");
 
     __shared__ __attribute__((aligned(16))) char q_lds[WIDE_ROWS * G::QSTR];
@@ -200,6 +209,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rw = wv % NRW;                    // which rows
+    const int par = wv / NRW;                   // which tile of a step
     const int n = lane & 15;
     const int q = lane >> 4;
     HW_MARK(8);
@@ -271,29 +282,37 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         }
     }
     const int r0 = rg * WIDE_ROWS;              // first row of the workgroup
-    const int w0 = r0 + wv * WROWS;             // first row of this wave
+    const int w0 = r0 + rw * WROWS;             // first row of this wave
     const int GQ = a.Hq / a.Hkv;
-
-    unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
-    int f = 0, L = 0, lt0 = 0, lt1 = 0;
-    bool opens_fragment = false;
-    u32x4 view = {0, 0, 0, 0};                               // this wave's image of the current fragment (K or V slice)
-    QueryRotation<DT, E, WIDE_ROWS, G::QSTR, PRE, NT> qrot;     // pre-rotated queries, or too many (worker, token) pairs for the staged tables
-    WRot wrot;
     // (worker, token) pairs the rows of this workgroup belong to
     const int ws_lo = fast_div(r0, a.magic_gq);
     const int nws = fast_div(min(r0 + WIDE_ROWS, a.R) - 1, a.magic_gq) - ws_lo + 1;
     const bool staged = !PRE && nws <= WRot::CSMAX;          // uniform over the workgroup
+    // The queries to rotate are the same for every fragment: they are requested here, before the workgroup's tile range
+    // and first fragment are worked out, and are on their way while that happens.
+    WRot wrot;
+    const bool early_queries = staged;
+    if (early_queries) wrot.load_queries(a, hkv, r0, GQ, tid);
+
+    HW_MARK(10);
+    unsigned long long todo = __ballot(lane < a.F && max(T0, my_tb) < min(T1, my_te));
+    int f = 0, L = 0, lt0 = 0, lt1 = 0;
+    bool opens_fragment = false;
+    u32x4 view = {0, 0, 0, 0};                               // this wave's image of the current fragment (K or V slice)
+    [[maybe_unused]] QueryRotation<DT, E, WIDE_ROWS, G::QSTR, true, NT> qrot;     // pre-rotated queries: a copy into LDS
     int lm = 0;
 
-    // this wave's share of tile `lt` (fragment-local) into ring slot `sl`; a tile that does not exist is requested out of
-    // range: the same number of transfers, no memory traffic, zeros in LDS
-    auto request = [&](int sl, int lt) {
-        const unsigned tile_bytes = (unsigned)(lt * TILE * image_row);
-        wide_request<TPW>(view, __builtin_amdgcn_readfirstlane(my_image + sl * SLOT), lt < lt1 ? tile_bytes : OOB_OFFSET, off);
+    // this wave's share of the PAR tiles of the step that starts at tile `lt` (fragment-local) into step slot `ss`; a tile
+    // that does not exist is requested out of range: the same number of transfers, no memory traffic, zeros in LDS
+    auto request = [&](int ss, int lt) {
+#pragma unroll
+        for (int pp = 0; pp < PAR; ++pp) {
+            const unsigned tile_bytes = (unsigned)((lt + pp) * TILE * image_row);
+            wide_request<TPW>(view, __builtin_amdgcn_readfirstlane(my_image + (ss * PAR + pp) * SLOT), lt + pp < lt1 ? tile_bytes : OOB_OFFSET, off);
+        }
     };
 
-    auto open_segment = [&]() {
+    auto open_segment = [&](bool queries_requested) {
         f = __builtin_ctzll(todo);
         todo &= todo - 1;
         const int fb = __builtin_amdgcn_readlane(my_tb, f);
@@ -307,38 +326,68 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         lt0 = s0 - fb;
         lt1 = s1 - fb;
         opens_fragment = s0 == fb;
-        // The first tile is requested before the queries: the compiler's wait for the query loads then also waits for it
-        // (loads complete in order), which costs nothing, the tile being needed first anyway.  The other look-ahead
-        // tiles follow after the rotation, so that the rotation does not wait for them as well.
+        // The first step is requested before the queries: the compiler's wait for the query loads then also waits for it
+        // (loads complete in order), which costs nothing, its tiles being needed first anyway.  The other look-ahead
+        // steps follow when the queries have arrived, so that the rotation does not wait for them as well.
         request(0, lt0);
-        if (!PRE && staged) wrot.load(a, f, hkv, r0, GQ, tid, ws_lo, nws);
-        else qrot.load(a, f, hkv, r0, GQ, tid);
+        HW_MARK(11);
+        // (the thread index as the compiler cannot see through it: what is derived from it -- rows, addresses of the
+        // queries -- is then formed per segment instead of once in front of the loop over the segments, from where it
+        // would stay in registers across the tile loops, which have none to spare)
+        int tids = tid;
+        asm volatile("" : "+v"(tids));
+        if constexpr (PRE) {
+            qrot.load(a, f, hkv, r0, GQ, tids);
+        } else if (staged) {
+            if (!queries_requested) wrot.load_queries(a, hkv, r0, GQ, tids);
+            wrot.load_tables(a, f, tids, ws_lo, nws);
+        }
         // the bound of row tid / TPR (TPR threads per row, all load: keeps the load unconditional)
-        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + tid / TPR, a.R - 1), a.magic_gq)];
+        lm = a.loc[(size_t)f * a.W * a.S + fast_div(min(r0 + tids / TPR, a.R - 1), a.magic_gq)];
     };
     bool more = todo != 0;
-    if (more) open_segment();
+    if (more) open_segment(early_queries);
     HW_MARK(6);
     bool hw_first = true;
 
     while (more) {
         __syncthreads();   // previous segment's readers are done with q_lds / lim_lds
         if (hw_first) HW_MARK(7);
+        int tids = tid;        // (see open_segment)
+        asm volatile("" : "+v"(tids));
+        // Every load of open_segment is waited for here, in a form the compiler sees: it waits for a load where its result
+        // is first used and counts only the loads it knows of, so a wait that it places further down -- for the bound
+        // below, the last load of open_segment -- would also wait for the look-ahead steps requested in between.
+        // (Nothing is lost: the queries are needed now, and the first step was requested before them.)
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+        int limv = (r0 + tids / TPR < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;   // by every thread, see paged_wide_kernel
+        asm volatile("" : "+v"(limv));
         if (!PRE && staged) {
-            wrot.stage(cs_lds, tid, nws);
-            // The barrier above has waited for every load of open_segment: the other look-ahead tiles can be requested
+            wrot.stage(cs_lds, tids, nws);
+            if (hw_first) HW_MARK(13);
+            // The barrier above has waited for every load of open_segment: the other look-ahead steps can be requested
             // here, ahead of the rotation arithmetic, which waits for nothing from memory any more.  (An LDS-only barrier
             // again: __syncthreads() would wait for the requests just issued.)
 #pragma unroll
-            for (int i = 1; i < D; ++i) request(i, lt0 + i);
+            for (int i = 1; i < DP; ++i) request(i, lt0 + i * PAR);
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            wrot.rotate(a, q_lds, cs_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid, ws_lo);
+            if (hw_first) HW_MARK(14);
+            wrot.rotate(a, q_lds, cs_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tids, ws_lo);
+        } else if constexpr (PRE) {
+            qrot.finish(a, q_lds, f, hkv, r0, GQ, false, tids);
         } else {
-            qrot.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tid);
+            // too many (worker, token) pairs for the staged tables (GQA ratio below 4): every row loads its own table row,
+            // here and not ahead of time in open_segment, so that the registers of this path are not held across the tile
+            // loops of the common one
+            QueryRotation<DT, E, WIDE_ROWS, G::QSTR, false, NT> qslow;
+            qslow.load(a, f, hkv, r0, GQ, tids);
+            qslow.finish(a, q_lds, f, hkv, r0, GQ, a.rq != nullptr && opens_fragment, tids);
+            // (said once more where the compiler sees it: without it, it takes this path's loads for outstanding on the
+            // other path of the next segment and waits there, in the middle of the rotation, for "everything")
+            __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         }
-        int limv = (r0 + tid / TPR < a.R) ? min(L, max(0, lm + 1)) : 0x7fffffff;   // by every thread, see paged_wide_kernel
-        asm volatile("" : "+v"(limv));
-        if (tid % TPR == 0) lim_lds[tid / TPR] = limv;
+        if (tids % TPR == 0) lim_lds[tids / TPR] = limv;
+        if (hw_first) HW_MARK(12);
         // q_lds and lim_lds become visible: a barrier for LDS only.  __syncthreads() would also wait for the stores of
         // the rotated queries to be acknowledged by memory, which nobody here depends on.
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -350,12 +399,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
             for (int j = 0; j < G::KJ; ++j)
-                qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (wv * WROWS + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
+                qreg[rb * G::KJ + j] = *reinterpret_cast<const u32x4*>(q_lds + (rw * WROWS + rb * 16 + n) * G::QSTR + (4 * j + q) * 16);
         int lim[RB];
         int maxlim = 0, minlim = 0x7fffffff;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
-            lim[rb] = lim_lds[wv * WROWS + rb * 16 + n];
+            lim[rb] = lim_lds[rw * WROWS + rb * 16 + n];
             const bool pad = w0 + rb * 16 + n >= a.R;
             maxlim = max(maxlim, pad ? 0 : lim[rb]);
             minlim = min(minlim, lim[rb]);
@@ -364,39 +413,41 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         minlim = __builtin_amdgcn_readfirstlane(row_min16(minlim));
         if (PRE || !staged) {
 #pragma unroll
-            for (int i = 1; i < D; ++i) request(i, lt0 + i);
+            for (int i = 1; i < DP; ++i) request(i, lt0 + i * PAR);
         }
 
         {
-            // Two loops, one instantiation of the tile arithmetic in each: first the tiles every row of this wave sees
+            // A step = PAR tiles behind one barrier, one for each of the waves that share their rows.  Two loops, one
+            // instantiation of the tile arithmetic in each: first the steps in which every row of this wave sees its tile
             // completely, then the rest.  With both instantiations in one loop body the compiler merges their accumulators
-            // through copies (48 v_mov_b64 per tile).  The waves of a workgroup may change loops at different tiles; each
-            // still passes one barrier per tile.
-            int sl = 0;                                   // ring slot of tile l
-            int l = lt0;
-            auto arrive = [&]() {                         // request tile l + D, wait for tile l
-                int rs = sl + D;
-                if (rs >= NS) rs -= NS;
-                request(rs, l + D);
-                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(D * TPW) : "memory");
+            // through copies (48 v_mov_b64 per tile).  The waves of a workgroup may change loops at different steps; each
+            // still passes one barrier per step.
+            int ss = 0;                                   // step slot of the current step
+            int l = lt0;                                  // its first tile
+            auto arrive = [&]() {
+                // this wave's transfers of the step have landed (the DP - 1 steps requested since may stay in flight: loads
+                // complete in order), then every wave's.  Behind the barrier the slots of the step before are free:
+                // request step + DP into them.
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((DP - 1) * TPS) : "memory");
+                request(ss == 0 ? NSTEP - 1 : ss - 1, l + DP * PAR);
                 if (hw_first) { HW_MARK(2); hw_first = false; }
             };
             const int lfast = maxlim > 0 ? min(lt1, minlim / TILE) : lt0;
 #pragma unroll 1
-            for (; l < lfast; ++l) {
+            for (; l + par < lfast; l += PAR) {
                 arrive();
-                const char* slot = ring + sl * SLOT;
-                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
-                sl = sl + 1 == NS ? 0 : sl + 1;
+                const char* slot = ring + (ss * PAR + par) * SLOT;
+                compute_tile<DT, E, EV, RB, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (l + par) * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
+                ss = ss + 1 == NSTEP ? 0 : ss + 1;
             }
 #pragma unroll 1
-            for (; l < lt1; ++l) {
+            for (; l < lt1; l += PAR) {
                 arrive();
-                if (l * TILE < maxlim) {
-                    const char* slot = ring + sl * SLOT;
-                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, l * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
+                if (l + par < lt1 && (l + par) * TILE < maxlim) {
+                    const char* slot = ring + (ss * PAR + par) * SLOT;
+                    compute_tile<DT, E, EV, RB, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (l + par) * TILE, n, q, a.sc, slot, slot + KBYTES, voff);
                 }
-                sl = sl + 1 == NS ? 0 : sl + 1;
+                ss = ss + 1 == NSTEP ? 0 : ss + 1;
             }
         }
         // the requests behind the last tile (they fetched nothing) must have landed before the ring is used again
@@ -404,23 +455,54 @@ __global__ __launch_bounds__(NW * 64, 1) void attention_wide_kernel(const Kernel
         more = todo != 0;
         if (more) {
             __syncthreads();   // every wave is done with the ring
-            open_segment();
+            open_segment(false);
         }
     }
 
-    // ---- every wave stores the partial of its own rows.  The accumulator layout scatters a row over the lanes in 16-byte
-    // pieces; written like that, a partial (17 MB per launch at 128 rows x 32 workgroups x 8 heads) would reach memory as
-    // a million partial-line writes.  So each 16-row block goes through LDS once -- a piece of the ring, which no tile
-    // needs any more -- and leaves as whole rows, 1 KB per store. ----
+    // ---- The PAR waves that share their rows hold a partial sum each: block rb of the rows goes to wave rb % PAR of them
+    // through LDS, lane for lane in the accumulator layout, and is added up there.  Then every wave stores the blocks it
+    // owns.  The accumulator layout scatters a row over the lanes in 16-byte pieces; written like that, a partial (17 MB
+    // per launch at 128 rows x 32 workgroups x 8 heads) would reach memory as a million partial-line writes.  So each
+    // 16-row block goes through LDS once more -- all of this in the ring, which no tile needs any more -- and leaves as
+    // whole rows, 1 KB per store. ----
     {
         constexpr int OSTR = EV + 4;                                  // floats per staged row (padded against bank conflicts)
-        static_assert(NW * 16 * OSTR * 4 <= NS * SLOT, "one 16-row block per wave fits into the ring");
+        constexpr int REGION = 16 * OSTR;                             // floats per wave: a staged 16-row block, or a block in accumulator layout
+        static_assert(G::NOC * 64 * 4 <= REGION && (NW * REGION + NW * 64 * 2) * 4 <= NS * SLOT, "the blocks of all waves fit into the ring");
         HW_MARK(3);
         __syncthreads();                                              // every wave has left the last tile
         HW_MARK(4);
-        float* stage = reinterpret_cast<float*>(ring) + wv * 16 * OSTR;
+        float* const regions = reinterpret_cast<float*>(ring);
+        float* const mls = regions + NW * REGION;
+        if constexpr (PAR > 1) {
+#pragma unroll
+            for (int rb = 0; rb < RB; ++rb) {
+                const int owner = rw + (rb % PAR) * NRW;
+                if (owner != wv) {
+#pragma unroll
+                    for (int c = 0; c < G::NOC; ++c) *reinterpret_cast<f32x4*>(regions + owner * REGION + (c * 64 + lane) * 4) = st.o[rb][c];
+                    *reinterpret_cast<f32x2*>(mls + (owner * 64 + lane) * 2) = f32x2{st.m[rb], st.l[rb]};
+                }
+            }
+            __syncthreads();
+        }
+        float* stage = regions + wv * REGION;
 #pragma unroll
         for (int rb = 0; rb < RB; ++rb) {
+            if (rw + (rb % PAR) * NRW != wv) continue;                // uniform over the wave
+            if constexpr (PAR > 1) {
+                const f32x2 oml = *reinterpret_cast<const f32x2*>(mls + (wv * 64 + lane) * 2);
+                const float mnew = fmaxf(st.m[rb], oml.x);
+                const float mine = exp2f(st.m[rb] - mnew), theirs = exp2f(oml.x - mnew);
+#pragma unroll
+                for (int c = 0; c < G::NOC; ++c) {
+                    const f32x4 o2 = *reinterpret_cast<const f32x4*>(stage + (c * 64 + lane) * 4);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) st.o[rb][c][i] = st.o[rb][c][i] * mine + o2[i] * theirs;
+                }
+                st.l[rb] = st.l[rb] * mine + oml.y * theirs;
+                st.m[rb] = mnew;
+            }
             const float lsum = quarter_sum(st.l[rb]);
             const int row0 = w0 + rb * 16;                            // first row of the block
             const size_t prow0 = (size_t)(hkv * a.slot_stride + g) * a.R + row0;
@@ -484,10 +566,6 @@ struct PlanSlot {
     int w, rg, qs, qe, split, ns;
     bool found;
 };
-#ifndef HW_PLAN_W_HEAVY
-#define HW_PLAN_W_HEAVY 4
-#define HW_PLAN_W_LIGHT 3
-#endif
 template <int NTW>
 __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, int hkv, int GQ, int T, int tid) {
     constexpr int NT = PLAN_MAX_GROUPS;     // threads that take part (the others only meet the barriers)
@@ -567,7 +645,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
         gw = grp_w[tid];
         grg = grp_rg[tid];
         rows = min((seq_qe[gw] - seq_qs[gw]) * GQ - grg * WIDE_ROWS, WIDE_ROWS);
-        work = seq_tiles[gw] * (rows > WIDE_ROWS / 2 ? HW_PLAN_W_HEAVY : HW_PLAN_W_LIGHT);
+        work = seq_tiles[gw] * (rows > WIDE_ROWS / 2 ? 4 : 3);
         most = max(1, seq_tiles[gw] / 4);
     }
     // One slot each, and the other pslots - G in proportion to the work (rounded down, so they fit; the quotient in
@@ -642,7 +720,7 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     constexpr int TPS = PAR * TPW;               // transfers a wave issues per step
     constexpr int SLOT = KBYTES + VBYTES;
     constexpr int RPL = 64 / G::CPR;             // tile rows one transfer covers
-    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (KBYTES / 1024) % TPW == 0 && NS % PAR == 0 && DP >= 2 && G::KROW == G::VROW &&
+    static_assert(G::SZ == 2 && KBYTES == VBYTES && TPW >= 1 && (2 * KBYTES / 1024) % TPW == 0 && NS % PAR == 0 && DP >= 1 && G::KROW == G::VROW &&
                       NW % PAR == 0 && (PAR == 1 || PAR == 2) && RB >= 1,
                   "16-bit types; a wave's transfers belong to one image");
 
@@ -654,7 +732,7 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     constexpr int RING_BYTES = NS * SLOT > QOFF + QBYTES ? NS * SLOT : QOFF + QBYTES;
     __shared__ int lim_lds[WIDE_ROWS];
     __shared__ int bt_lds[PAGED_WIDE_MAX_BLOCKS];
-    __shared__ __attribute__((aligned(256))) char ring[RING_BYTES];
+    __shared__ __attribute__((aligned(16))) char ring[RING_BYTES];
     char* const q_lds = ring + QOFF;
 
     const int tid = threadIdx.x;
@@ -668,20 +746,30 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     HW_MARK(8);
     PagedHeaderBits hb;
     paged_header_request(hb);
-    // this wave's share of a tile's transfers: the first half of the waves fill the K image, the second half V
-    const bool k_wave = wv < NW / 2;
-    const int first = (k_wave ? wv : wv - NW / 2) * TPW;
+    // This wave's share of a tile's transfers.  With an even number of them a wave brings the same rows of both images:
+    // a row of the K cache and the row of the V cache with the same number lie at the same place of their caches, so one
+    // block look-up serves two transfers.  Otherwise the first half of the waves fill the K image, the second half V.
+    constexpr bool BOTH = TPW % 2 == 0;
+    constexpr int NI = BOTH ? 2 : 1;              // images a wave fills
+    constexpr int NP = TPW / NI;                  // 1 KB pieces of each
+    static_assert((KBYTES / 1024) % NP == 0 && NW * NP * NI * 1024 == KBYTES + VBYTES, "the waves' pieces tile both images");
+    const bool k_wave = BOTH || wv < NW / 2;
+    const int first = (BOTH ? wv : (k_wave ? wv : wv - NW / 2)) * NP;
     const int lrow = lane / G::CPR, lslot = lane % G::CPR;
-    unsigned chunk[TPW];                          // byte offset of this lane's 16 bytes within its row, per transfer
-    int trow[TPW];                                // the tile row it belongs to
+    unsigned chunk[NI][NP];                       // byte offset of this lane's 16 bytes within its row, per image and piece
+    int trow[NP];                                 // the tile row it belongs to
 #pragma unroll
-    for (int j = 0; j < TPW; ++j) {
+    for (int j = 0; j < NP; ++j) {
         const int row = (first + j) * RPL + lrow;
         const int key = G::CPR >= 16 ? (row & 15) : ((row >> 1) & (G::CPR - 1));
+        const unsigned kchunk = (unsigned)((lslot ^ key) << 4), vchunk = (unsigned)((lslot ^ (2 * vimg_segment_key<G::VROW>(row))) << 4);
         trow[j] = row;
-        chunk[j] = (unsigned)((k_wave ? (lslot ^ key) : (lslot ^ (2 * vimg_segment_key<G::VROW>(row)))) << 4);
+        chunk[0][j] = k_wave ? kchunk : vchunk;
+        if constexpr (BOTH) chunk[1][j] = vchunk;
     }
-    const unsigned my_image = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
+    unsigned my_image[NI];                        // where the pieces go in ring slot 0
+    my_image[0] = lds_address(ring) + (k_wave ? 0 : KBYTES) + first * 1024;
+    if constexpr (BOTH) my_image[1] = my_image[0] + KBYTES;
     unsigned voff[G::NOC];                             // this lane's positions in a V image (transposed reads)
     vtr_lane_offsets<G::VROW>(voff, lane);
     const PagedDevHeader ph = paged_header_wait(hb);
@@ -726,7 +814,9 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     if (r0 >= rend) return;                     // uniform over the workgroup
     const int cap = ph.block_size * ph.max_blocks;
     const HW_GLOBAL int* btw = ph.block_table + (size_t)w * ph.max_blocks;
-    const unsigned long long image = reinterpret_cast<unsigned long long>(k_wave ? ph.kcache : ph.vcache);
+    unsigned long long image[NI];
+    image[0] = reinterpret_cast<unsigned long long>(k_wave ? ph.kcache : ph.vcache);
+    if constexpr (BOTH) image[1] = reinterpret_cast<unsigned long long>(ph.vcache);
 
     DevHeader a;
     a.q = ph.q;
@@ -830,20 +920,25 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
 #pragma unroll
                     for (int pp = 0; pp < PAR; ++pp)
 #pragma unroll
-                        for (int j = 0; j < TPW; ++j) {
+                        for (int j = 0; j < NP; ++j) {
                             const int tok = min((tb + pp * ns) * TILE + trow[j], wgmax - 1);
                             const int bi = fast_div(tok, ph.magic_bs);
                             const int blk = min(max(bt_lds[bi], 0), ph.num_blocks - 1);
                             const int rid = (blk * ph.Hkv + hkv) * ph.block_size + (tok - bi * ph.block_size);
-                            src[pp * TPW + j] = image + (unsigned long long)(unsigned)rid * G::KROW + chunk[j];
+#pragma unroll
+                            for (int im = 0; im < NI; ++im)
+                                src[(pp * NP + j) * NI + im] = image[im] + (unsigned long long)(unsigned)rid * G::KROW + chunk[im][j];
                         }
                 };
                 auto request = [&](int step_slot, const unsigned long long* src) {
 #pragma unroll
                     for (int pp = 0; pp < PAR; ++pp)
 #pragma unroll
-                        for (int j = 0; j < TPW; ++j)
-                            lds_transfer_flat(__builtin_amdgcn_readfirstlane(my_image + (step_slot * PAR + pp) * SLOT + j * 1024), src[pp * TPW + j]);
+                        for (int j = 0; j < NP; ++j)
+#pragma unroll
+                            for (int im = 0; im < NI; ++im)
+                                lds_transfer_flat(__builtin_amdgcn_readfirstlane(my_image[im] + (step_slot * PAR + pp) * SLOT + j * 1024),
+                                                  src[(pp * NP + j) * NI + im]);
                 };
 
                 if (wgmax > 0) {   // uniform over the workgroup
@@ -880,7 +975,7 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
                     for (; tb + par * ns < tfast; tb += tstep) {
                         arrive();
                         const char* slot = ring + (sl * PAR + par) * SLOT;
-                        compute_tile<DT, E, EV, RBX, false, true, false, true, (RBX > 1)>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                        compute_tile<DT, E, EV, RBX, false, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                         sl = sl + 1 == NSTEP ? 0 : sl + 1;
                     }
 #pragma unroll 1
@@ -888,7 +983,7 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
                         arrive();
                         if ((tb + par * ns) * TILE < maxlim) {
                             const char* slot = ring + (sl * PAR + par) * SLOT;
-                            compute_tile<DT, E, EV, RBX, true, true, false, true, (RBX > 1)>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
+                            compute_tile<DT, E, EV, RBX, true, true, false, true>(TileRegs<DT, E, EV>(), q_lds, qreg, lim, st, (tb + par * ns) * TILE, n, q, ph.sc, slot, slot + KBYTES, voff);
                         }
                         sl = sl + 1 == NSTEP ? 0 : sl + 1;
                     }
@@ -964,21 +1059,27 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     else run(std::integral_constant<int, RB>{});
 }
 
-// Waves per workgroup.  Four waves of 32 rows each are the measured choice: eight waves of 16 rows (two per SIMD, the
-// usual cure for a loop that waits) double what the waves read out of LDS per tile, and the kernel got slower by a
-// tenth (27.3 against 24.7 us at 128 rows x 16 K tokens x 8 kv heads, fp16).
-constexpr int WIDE_WAVES = 4;
+// Waves per workgroup, how many of them share their rows, and ring slots (see PAGED_WIDE_WAVES for the layout).
+#ifndef HW_WIDE_WAVES
+#define HW_WIDE_WAVES 8
+#define HW_WIDE_PAR 2
+#define HW_WIDE_SLOTS 6
+#endif
+constexpr int WIDE_WAVES = HW_WIDE_WAVES;
+constexpr int WIDE_PAR = HW_WIDE_PAR;
+constexpr int WIDE_SLOTS = HW_WIDE_SLOTS;
 
 template <class DT>
 static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
-    constexpr int NS = 5;
+    constexpr int NS = WIDE_SLOTS;
     constexpr int NW = WIDE_WAVES;
+    constexpr int PAR = WIDE_PAR;
     if (ka.h.flags & KH_PREROTATED) {
-        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
-        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
     } else {
-        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, false, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
-        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, false, NW>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, false, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
+        else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, false, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
     }
     return hipGetLastError();
 }
@@ -999,9 +1100,9 @@ hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStre
 // 1/1/1/64, 16 x 4, 64 x 4, 25 x 4 and 12 x 4 query tokens, against eight waves of 16 rows that all take every tile (which
 // doubles what is read out of LDS per tile and row): 57.9 / 48.2 / 42.3 / 110.0 / 47.3 / 40.1 us against 64.7 / 52.4 / 43.4 /
 // 116.4 / 50.6 / 39.2 us; that form had in turn been 4 % faster than four waves of 32 rows on every tile (one per SIMD).
-// Ring of six 16 KB slots = three steps: one being multiplied, two in flight.  The two-block instantiation fits the 256
-// registers of a wave exactly (see LEAN in compute_tile); a spill there costs more than the registers it frees, because
-// the compiler's wait for the reload also waits for the tile transfers in flight.
+// Ring of six 16 KB slots = three steps: one being multiplied, two in flight.  The two-block instantiation has to fit the
+// 256 registers of a wave: a spill costs more than the registers it frees, because the compiler's wait for the reload
+// also waits for the tile transfers in flight.
 #ifndef HW_PAGED_WIDE_PAR
 #define HW_PAGED_WIDE_PAR 2
 #endif

@@ -60,20 +60,36 @@ def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp
         for label, block in zip(parts[1::2], parts[2::2]):
             if "Depth=2" not in block:
                 continue                                   # not inside a tile loop (the loop over fragments / segments is depth 1)
-            # a wave issues E / (8 * waves) transfers per tile (K + V bytes of a tile / 1 KB / waves); head dimension, ring
-            # slots, waves and the tiles per step from the name
-            m = re.search(r"attention_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELb[01]ELi(\d+)E", name)
-            if m:       # three tiles requested ahead of the one that is waited for
-                e, ns, nw = (int(x) for x in m.groups())
-                ahead = (ns - 2) * e // (8 * nw)
-            else:       # steps of `par` tiles, requested behind the barrier: one step stays in flight
-                m = re.search(r"paged_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELi(\d+)ELi(\d+)E", name)
-                assert m, name
-                e, ns, nw, par = (int(x) for x in m.groups())
-                ahead = (ns // par - 2) * par * e // (8 * nw)
+            # a wave issues E / (8 * waves) transfers per tile (K + V bytes of a tile / 1 KB / waves), a step is `par` tiles
+            # requested behind the barrier, and one step stays in flight; head dimension, ring slots, waves and tiles per
+            # step from the name
+            m = re.search(r"attention_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELb[01]ELi(\d+)ELi(\d+)E", name) or \
+                re.search(r"paged_wide_kernel\S*?ELi(\d+)ELi\d+ELi(\d+)ELi(\d+)ELi(\d+)E", name)
+            assert m, name
+            e, ns, nw, par = (int(x) for x in m.groups())
+            ahead = (ns // par - 2) * par * e // (8 * nw)
             assert ahead >= 1, name
             assert "scratch_" not in block, f"{name} {label}: scratch memory inside a tile loop"
             for m in re.finditer(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", block):
                 checked += 1
                 assert int(m.group(1)) >= ahead, f"{name} {label}: {m.group(0)} inside a tile loop"
     assert checked >= 2 * len(kernels)                    # every kernel has its own hand-counted waits there
+    # Outside the tile loops: a wait the COMPILER places (outside the inline-assembly brackets) behind transfers of the
+    # same block must leave those in flight -- the rotation of the queries runs beside the look-ahead steps requested just
+    # before it.
+    for name in kernels:
+        body = text[text.index(name + ":"):]
+        body = body[:body.index("; -- End function")]
+        parts = re.split(r"\n(\.LBB\d+_\d+):", body)
+        for label, block in zip(["entry"] + parts[1::2], parts[0::2]):
+            issued, in_asm = 0, False
+            for line in block.splitlines():
+                if "#ASMSTART" in line:
+                    in_asm = True
+                elif "#ASMEND" in line:
+                    in_asm = False
+                elif re.search(r"(buffer_load_dwordx4|global_load_lds_dwordx4)[^\n]*\b(lds|nt)\b", line) and in_asm:
+                    issued += 1
+                elif not in_asm:
+                    m = re.search(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", line)
+                    assert not (m and issued and int(m.group(1)) < issued), f"{name} {label}: {line.strip()} behind {issued} transfers"
