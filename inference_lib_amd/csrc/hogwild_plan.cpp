@@ -73,12 +73,12 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     const int rows = (int)rows_ll;
     plan->rows = rows;
     // up to 16 rows: one 16-row block per workgroup (two workgroups per CU); up to 96: two blocks, rows beyond 32 in
-    // further row groups that read the same KV; more: 128-row workgroups whose four waves share every K/V tile through
+    // further row groups that read the same KV; more: 128-row workgroups whose waves share every K/V tile through
     // LDS (16-bit types, lengths known on the host) -- a CU can take in about 16 B/clk, so what counts is that every
     // CU reads every byte once
     const bool wide_ok = p->dtype != HW_F32 && p->len_dev == nullptr && p->variant == HW_VARIANT_MFMA;
     plan->row_blocks = rows <= 16 ? 1 : 2;
-    if (wide_ok && rows > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;   // measured crossover: 80 rows 24.6 (narrow) / 25.6 us, 120 rows 28.0 / 27.4 us
+    if (wide_ok && rows > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;   // measured crossover: 95 rows 19.2 (narrow) / 19.9 us, 120 rows 21.8 / 20.6 us
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rows_per_wg = 16 * plan->row_blocks;
@@ -102,7 +102,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
         const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32) ? 2 : 1;
         const int target = per_cu * num_cus;
         wgs = target / (p->Hkv * plan->row_groups);
-        // narrow kernels deal a workgroup's tiles to its four waves; in the wide kernel every wave takes every tile
+        // narrow kernels deal a workgroup's tiles to its four waves; in the wide kernel the whole workgroup takes every tile
         const int by_work = wide ? (int)((tiles + 3) / 4) : (int)((tiles + hw::NWAVES - 1) / hw::NWAVES);
         if (wgs > by_work) wgs = by_work;
         // Small problems in 16-bit types: one workgroup per kv head (and row group) holds whole rows, writes the result
