@@ -1059,15 +1059,13 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     else run(std::integral_constant<int, RB>{});
 }
 
-// Waves per workgroup, how many of them share their rows, and ring slots (see PAGED_WIDE_WAVES for the layout).
-#ifndef HW_WIDE_WAVES
-#define HW_WIDE_WAVES 8
-#define HW_WIDE_PAR 2
-#define HW_WIDE_SLOTS 6
-#endif
-constexpr int WIDE_WAVES = HW_WIDE_WAVES;
-constexpr int WIDE_PAR = HW_WIDE_PAR;
-constexpr int WIDE_SLOTS = HW_WIDE_SLOTS;
+// Waves per workgroup, how many of them share their rows, and ring slots (see PAGED_WIDE_WAVES for the layout).  On the
+// multi-token benchmark workload (128 rows x 16 K tokens x 8 kv heads, fp16) four waves that take every tile measure the
+// same with the same prologue (ring of 4 slots: 20.2-20.4 us against 20.3-20.8 us on one box): there the tile loop runs at
+// the pace of the tile stream either way.
+constexpr int WIDE_WAVES = 8;
+constexpr int WIDE_PAR = 2;
+constexpr int WIDE_SLOTS = 6;
 
 template <class DT>
 static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream) {
@@ -1103,15 +1101,9 @@ hipError_t launch_attention_wide(const KernelArgs& ka, int dtype, int E, hipStre
 // Ring of six 16 KB slots = three steps: one being multiplied, two in flight.  The two-block instantiation has to fit the
 // 256 registers of a wave: a spill costs more than the registers it frees, because the compiler's wait for the reload
 // also waits for the tile transfers in flight.
-#ifndef HW_PAGED_WIDE_PAR
-#define HW_PAGED_WIDE_PAR 2
-#endif
-#ifndef HW_PAGED_WIDE_SLOTS
-#define HW_PAGED_WIDE_SLOTS 6
-#endif
 constexpr int PAGED_WIDE_WAVES = 8;
-constexpr int PAGED_WIDE_PAR = HW_PAGED_WIDE_PAR;
-constexpr int PAGED_WIDE_SLOTS = HW_PAGED_WIDE_SLOTS;
+constexpr int PAGED_WIDE_PAR = 2;
+constexpr int PAGED_WIDE_SLOTS = 6;
 
 template <class DT>
 static hipError_t launch_paged_wide_dt(const PagedHeader& ph, int E, hipStream_t stream) {
