@@ -203,6 +203,21 @@ def test_varlen_mixed_1_8_32_64_query_tokens():
     check(c, row_blocks=2)
 
 
+def test_paged_decode_full_size_of_the_benchmark():
+    """The paged decode benchmark workload at its full size (four sequences of 12 528 tokens, one query token each)."""
+    c = build_paged("bf16", 1, 4, 40, 8, 128, 16, 784, seq_lens=[12528] * 4, S=1, seed=63)
+    check(c)
+
+
+def test_varlen_full_size_of_the_benchmark():
+    """The packed-query benchmark workload at its full size (four sequences of 12 528 tokens with 1 / 8 / 32 / 64 query
+    tokens, QwQ-32B head shape, blocks of 16): the launch planned on the device against the oracle, and the 32-row kernel
+    (another kernel, another split, another order of summation) against the same oracle."""
+    c = build_paged("bf16", 1, 4, 40, 8, 128, 16, 784, seq_lens=[12528] * 4, q_lens=[1, 8, 32, 64], seed=62)
+    check(c)
+    check(c, row_blocks=2)
+
+
 def test_varlen_tokens_behind_the_last_sequence_give_zeros():
     """total_q may exceed cu_seqlens_q[-1]: the tokens behind the last sequence belong to none.  The device-planned launch
     gives them zeros (lse -inf); the other launches leave them unspecified, like the reference, but must get the tokens of
