@@ -566,6 +566,96 @@ struct PlanSlot {
     int w, rg, qs, qe, split, ns;
     bool found;
 };
+// Where the merge finds the partial sums of a row: {first slot | slots << 16, row within the slot}, written by the
+// workgroup that holds a row group's first slot; rows behind the last sequence (its query range ends at last_qe) have
+// none: the workgroup of slot 0 writes zeros for them, and the merge gives them zeros.
+template <int NTW>
+__device__ __forceinline__ void plan_row_table(const PagedDevHeader& ph, const PlanSlot& r, int item, int hkv, int GQ, int tid, int last_qe) {
+    HW_GLOBAL int* row_tab = reinterpret_cast<HW_GLOBAL int*>(ph.part_ml + (size_t)ph.Hkv * ph.nitems * PLAN_SLOT_ROWS * 2) + (size_t)hkv * ph.R * 2;
+    if (r.found && r.split == 0) {
+        const int nrows = min((r.qe - r.qs) * GQ - r.rg * WIDE_ROWS, WIDE_ROWS);
+        const int row = r.qs * GQ + r.rg * WIDE_ROWS + tid;
+        if (tid < nrows && row < ph.R) {
+            row_tab[2 * row] = (item - r.split) | (r.ns << 16);
+            row_tab[2 * row + 1] = tid;
+        }
+    }
+    if (item == 0) {
+        const int covered = min(last_qe * GQ, ph.R);
+        for (int i = covered * 2 + tid; i < ph.R * 2; i += NTW) row_tab[i] = 0;
+    }
+}
+
+// The same plan for launches of at most 64 sequences and 64 slots per kv head, worked out by every wave for itself with
+// cross-lane operations (lane = sequence, then lane = row group): no LDS, no barriers.  (The general form below meets
+// sixteen workgroup barriers; on four sequences it took 2.6 us of every workgroup's prologue.)
+__device__ __forceinline__ int wave_scan_inclusive(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);    // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);    // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);    // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);    // row_shr:8: inclusive within rows of 16 lanes
+    v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);    // row_bcast:15 into rows 1 and 3
+    v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);    // row_bcast:31 into rows 2 and 3
+    return v;
+}
+template <int NTW>
+__device__ __forceinline__ PlanSlot plan_slot_wave(const PagedDevHeader& ph, int item, int hkv, int GQ, int T, int tid) {
+    const int lane = tid & 63;
+    const int pslots = ph.nitems;
+    const int cap = ph.block_size * ph.max_blocks;
+    // lane = sequence
+    int qs = 0, qe = 0, tiles = 0, cnt = 0;
+    if (lane < ph.W) {
+        qs = min(max(ph.cu_q[lane], 0), T);
+        qe = min(max(ph.cu_q[lane + 1], qs), T);
+        int len = 0;
+        for (int f = 0; f < ph.F; ++f) len = max(len, ph.frag_len[f * ph.W + lane]);
+        len = min(len, cap);
+        tiles = (len + TILE - 1) / TILE;
+        cnt = ((qe - qs) * GQ + WIDE_ROWS - 1) / WIDE_ROWS;
+    }
+    const int gend = wave_scan_inclusive(cnt);          // row groups up to and including this sequence
+    const int G = min(__builtin_amdgcn_readlane(gend, 63), min(64, pslots));
+    // lane = row group: its sequence is the first whose groups reach beyond it
+    int w = 0;
+    for (int sq = 0; sq < ph.W; ++sq) w += __builtin_amdgcn_readlane(gend, sq) <= lane ? 1 : 0;
+    w = min(w, ph.W - 1);
+    const int w_gend = __shfl(gend, w, 64), w_cnt = __shfl(cnt, w, 64), w_qs = __shfl(qs, w, 64), w_qe = __shfl(qe, w, 64);
+    const int w_tiles = __shfl(tiles, w, 64);
+    const bool valid = lane < G;
+    const int rg = lane - (w_gend - w_cnt);
+    const int rows = min((w_qe - w_qs) * GQ - rg * WIDE_ROWS, WIDE_ROWS);
+    const int work = valid ? w_tiles * (rows > WIDE_ROWS / 2 ? 4 : 3) : 0;
+    const int most = max(1, w_tiles / 4);
+    auto wave_total = [&](int v) { return __builtin_amdgcn_readlane(wave_scan_inclusive(v), 63); };
+    // one slot each, and the other pslots - G in proportion to the work (see plan_slot)
+    const int all_work = wave_total(work);
+    const float share = (float)(pslots - G) * (1.0f - 1.0f / (1 << 20)) * __builtin_amdgcn_rcpf((float)max(all_work, 1));
+    int n = valid ? min(1 + (int)((float)work * share), most) : 0;
+    const int left = pslots - wave_total(n);
+    const int load = (valid && n < most) ? __float_as_int((float)work * __builtin_amdgcn_rcpf((float)n)) : -1;
+    int ahead = 0;
+    for (int g = 0; g < G; ++g) {
+        const int lg = __builtin_amdgcn_readlane(load, g);
+        ahead += (lg > load || (lg == load && g < lane)) ? 1 : 0;
+    }
+    if (load >= 0 && ahead < left) ++n;
+    const int slot0 = wave_scan_inclusive(n) - n;
+    n = max(min(n, pslots - slot0), 0);                 // (cannot bite)
+    const unsigned long long owner = __ballot(valid && item >= slot0 && item < slot0 + n);
+    PlanSlot r;
+    r.found = owner != 0;
+    const int l = r.found ? __builtin_ctzll(owner) : 0;
+    r.w = __builtin_amdgcn_readlane(w, l);
+    r.rg = __builtin_amdgcn_readlane(rg, l);
+    r.qs = __builtin_amdgcn_readlane(w_qs, l);
+    r.qe = __builtin_amdgcn_readlane(w_qe, l);
+    r.split = item - __builtin_amdgcn_readlane(slot0, l);
+    r.ns = __builtin_amdgcn_readlane(n, l);
+    plan_row_table<NTW>(ph, r, item, hkv, GQ, tid, __builtin_amdgcn_readlane(qe, ph.W - 1));
+    return r;
+}
+
 template <int NTW>
 __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds, int item, int hkv, int GQ, int T, int tid) {
     constexpr int NT = PLAN_MAX_GROUPS;     // threads that take part (the others only meet the barriers)
@@ -675,23 +765,7 @@ __device__ __forceinline__ PlanSlot plan_slot(const PagedDevHeader& ph, int* lds
     PlanSlot r;
     r.w = shared[1]; r.rg = shared[2]; r.qs = shared[3]; r.qe = shared[4]; r.split = shared[5]; r.ns = shared[6];
     r.found = r.w >= 0;
-    // where the merge finds the partial sums of a row: {first slot | slots << 16, row within the slot}; rows behind the
-    // last sequence have none (the merge writes zeros for them)
-    {
-        HW_GLOBAL int* row_tab = reinterpret_cast<HW_GLOBAL int*>(ph.part_ml + (size_t)ph.Hkv * pslots * PLAN_SLOT_ROWS * 2) + (size_t)hkv * ph.R * 2;
-        if (r.found && r.split == 0) {
-            const int nrows = min((r.qe - r.qs) * GQ - r.rg * WIDE_ROWS, WIDE_ROWS);
-            const int row = r.qs * GQ + r.rg * WIDE_ROWS + tid;
-            if (tid < nrows && row < ph.R) {
-                row_tab[2 * row] = (item - r.split) | (r.ns << 16);
-                row_tab[2 * row + 1] = tid;
-            }
-        }
-        if (item == 0) {
-            const int covered = min(seq_qe[ph.W - 1] * GQ, ph.R);
-            for (int i = covered * 2 + tid; i < ph.R * 2; i += NTW) row_tab[i] = 0;
-        }
-    }
+    plan_row_table<NTW>(ph, r, item, hkv, GQ, tid, seq_qe[ph.W - 1]);
     return r;
 }
 
@@ -791,7 +865,9 @@ __global__ __launch_bounds__(NW * 64, 1) void paged_wide_kernel(const PagedHeade
     int w, rg, qs, qe, ns;
     size_t pbase;                           // row of the partial arrays that holds the workgroup's first row
     if (ph.flags & PH_PLANNED) {
-        const PlanSlot ps = plan_slot<NT>(ph, reinterpret_cast<int*>(ring), item, hkv, GQ, T, tid);   // (the ring is not in use yet)
+        const PlanSlot ps = (ph.W <= 64 && ph.nitems <= 64)      // uniform over the launch
+                                ? plan_slot_wave<NT>(ph, item, hkv, GQ, T, tid)
+                                : plan_slot<NT>(ph, reinterpret_cast<int*>(ring), item, hkv, GQ, T, tid);   // (the ring is not in use yet)
         if (!ps.found) return;              // a slot the plan left empty; uniform over the workgroup
         w = __builtin_amdgcn_readfirstlane(ps.w);
         rg = __builtin_amdgcn_readfirstlane(ps.rg);
