@@ -89,6 +89,10 @@ typedef enum hw_dtype { HW_F32 = 0, HW_F16 = 1, HW_BF16 = 2 } hw_dtype;
  *   row_blocks 0 = choose automatically; 1 or 2 = 16-row MFMA blocks per workgroup (rows beyond that are
  *              spread over more workgroups that read the same KV); 8 = 128-row workgroups whose waves share every K/V
  *              tile through LDS (16-bit types without len_dev; the automatic choice beyond 96 rows per kv head)
+ *   E, Ev      head dimensions: E == Ev in {64, 128, 256}, anything else returns HW_ERR_UNSUPPORTED (the reference's
+ *              kernel is a template over E and Ev and is instantiated for 128 only, src/kernels/kernel_v21.cuh:28,982).
+ *              Head dimension 256 exists with one 16-row block per workgroup (row_blocks is taken as 1) and without
+ *              the VALU-logits variant; the paged operators take it in the 16-bit types.
  *   variant    HW_VARIANT_MFMA (0, default): logits and output on the matrix cores.  HW_VARIANT_VALU_QK: the logits
  *              K.Q^T by VALU dot products (v_dot2_f32_bf16 / _f16, v_fma_f32) in the same kernel, the inner product the
  *              reference uses (src/kernels/kernel_v21.cuh:161-180); exists so that the matrix-core choice can be measured

@@ -474,7 +474,7 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
                 for (int rb = 0; rb < RB; ++rb) st.o[rb][c] = Elem<DT>::mfma(vop, pp[rb], st.o[rb][c]);
             }
         } else
-        // dword d of a lane's V row holds ev (n*EVL + 2d, n*EVL + 2d + 1); gather the 8 tokens of each ev.
+        // dword d of a lane's V row holds two consecutive ev (out_ev(2d, n) and the next); gather the 8 tokens of each ev.
 #pragma unroll
         for (int d = 0; d < G::VW; ++d) {
             u32x4 lo, hi;
@@ -509,7 +509,9 @@ __device__ __forceinline__ void compute_tile(const TileRegs<DT, E, EV>& t_in, co
 template <class DT, int EV>
 __device__ __forceinline__ int out_ev(int c, int i) {
     if constexpr (Elem<DT>::size == 2) {
-        return i * (EV / 16) + c;              // lane i of a V row holds EV/16 consecutive elements
+        // lane i of a V row holds EV/16 consecutive elements -- of each 256-byte half, when the row has two (EV = 256)
+        constexpr int CPL = EV / 16 > 8 ? 8 : EV / 16;
+        return (c / CPL) * (16 * CPL) + i * CPL + (c % CPL);
     } else {
         return (c >> 2) * 64 + i * 4 + (c & 3);  // 16 lanes x 4 floats per 256-byte load, c>>2 selects the load
     }

@@ -462,10 +462,22 @@ static hipError_t launch_attention_rb(const KernelArgs& ka, int rb, hipStream_t 
     return hipGetLastError();
 }
 
+// Head dimension 256: one 16-row block per workgroup and one wave per SIMD.  A K tile is 16 KB per wave, and two row
+// blocks of 256-wide accumulators next to the query operands and two V tiles do not fit the register file.
+template <class DT, bool PRE, bool DEVLEN>
+static hipError_t launch_attention_256(const KernelArgs& ka, int rb, hipStream_t stream) {
+    if (rb != 1) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((attention_kernel<DT, 256, 256, 1, 1, Elem<DT>::size == 2 ? 2 : 1, PRE, DEVLEN>), dim3(ka.h.nwg), dim3(NTHREADS), 0,
+                       stream, ka);
+    return hipGetLastError();
+}
+
 template <class DT>
 static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, int variant, hipStream_t stream) {
+    if (E != 64 && E != 128 && E != 256) return hipErrorInvalidValue;
     if (variant == HW_VARIANT_VALU_QK) {     // fused entry, one row block, lengths from the host (checked by the caller)
         constexpr bool half = Elem<DT>::size == 2;
+        if (E == 256) return hipErrorInvalidValue;
         if (E == 128)
             hipLaunchKernelGGL((attention_kernel<DT, 128, 128, 1, half ? 2 : 1, half ? 2 : 1, false, false, true>), dim3(ka.h.nwg),
                                dim3(NTHREADS), 0, stream, ka);
@@ -476,13 +488,16 @@ static hipError_t launch_attention_dt(const KernelArgs& ka, int E, int rb, int v
     }
     if (ka.h.flags & KH_PREROTATED) {
         if (ka.h.len_dev != nullptr) return hipErrorInvalidValue;   // device-resident lengths exist for the fused entry only
+        if (E == 256) return launch_attention_256<DT, true, false>(ka, rb, stream);
         if (E == 128) return launch_attention_rb<DT, 128, 128, true, false>(ka, rb, stream);
         return launch_attention_rb<DT, 64, 64, true, false>(ka, rb, stream);
     }
     if (ka.h.len_dev != nullptr) {
+        if (E == 256) return launch_attention_256<DT, false, true>(ka, rb, stream);
         if (E == 128) return launch_attention_rb<DT, 128, 128, false, true>(ka, rb, stream);
         return launch_attention_rb<DT, 64, 64, false, true>(ka, rb, stream);
     }
+    if (E == 256) return launch_attention_256<DT, false, false>(ka, rb, stream);
     if (E == 128) return launch_attention_rb<DT, 128, 128, false, false>(ka, rb, stream);
     return launch_attention_rb<DT, 64, 64, false, false>(ka, rb, stream);
 }
@@ -505,7 +520,12 @@ static hipError_t launch_merge_ev(const MergeArgs& ma, hipStream_t stream) {
         const int blocks = ma.Hkv * ((ma.R + RPW - 1) / RPW);
         hipLaunchKernelGGL((merge_kernel<DT, EV, RPW>), dim3(blocks), dim3(256), 0, stream, ma);
     };
-    if (ns <= 4 && NPG >= 8) go(std::integral_constant<int, 8>{});
+    bool eight = false;
+    if constexpr (NPG >= 8) {
+        eight = ns <= 4;
+        if (eight) go(std::integral_constant<int, 8>{});
+    }
+    if (eight) {}
     else if (ns <= 4 * (NPG / 4)) go(std::integral_constant<int, 4>{});
     else if (ns <= 4 * (NPG / 2)) go(std::integral_constant<int, 2>{});
     else go(std::integral_constant<int, 1>{});
@@ -514,6 +534,7 @@ static hipError_t launch_merge_ev(const MergeArgs& ma, hipStream_t stream) {
 
 template <class DT>
 static hipError_t launch_merge_dt(const MergeArgs& ma, int EV, hipStream_t stream) {
+    if (EV == 256) return launch_merge_ev<DT, 256>(ma, stream);
     if (EV == 128) return launch_merge_ev<DT, 128>(ma, stream);
     return launch_merge_ev<DT, 64>(ma, stream);
 }

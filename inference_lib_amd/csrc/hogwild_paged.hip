@@ -300,7 +300,16 @@ static hipError_t launch_paged_rb(const PagedHeader& ph, int rb, hipStream_t str
 
 template <class DT>
 static hipError_t launch_paged_dt(const PagedHeader& ph, int E, int rb, hipStream_t stream) {
+    if (E == 256) {     // one 16-row block per workgroup, one wave per SIMD; 16-bit types (two fp32 K tiles per wave exceed the LDS)
+        if constexpr (Elem<DT>::size == 2) {
+            if (rb != 1) return hipErrorInvalidValue;
+            hipLaunchKernelGGL((paged_attention_kernel<DT, 256, 256, 1, 1>), dim3(ph.nwg), dim3(NTHREADS), 0, stream, ph);
+            return hipGetLastError();
+        }
+        return hipErrorInvalidValue;
+    }
     if (E == 128) return launch_paged_rb<DT, 128, 128>(ph, rb, stream);
+    if (E != 64) return hipErrorInvalidValue;
     return launch_paged_rb<DT, 64, 64>(ph, rb, stream);
 }
 

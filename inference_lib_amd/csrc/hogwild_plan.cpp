@@ -56,7 +56,8 @@ int validate(const hw_problem* p, int fused) {
     if (!aligned16(p->out) || !aligned16(p->q)) return HW_ERR_ALIGN;
     if (fused && (!aligned16(p->cosines) || !aligned16(p->sines) || !aligned16(p->rq))) return HW_ERR_ALIGN;
     // kernels are instantiated for these head dims (never a silent no-op as in kernel_v21.cuh:992-995)
-    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
+    if (p->E != p->Ev || (p->E != 64 && p->E != 128 && p->E != 256)) return HW_ERR_UNSUPPORTED;
+    if (p->E == 256 && p->variant != HW_VARIANT_MFMA) return HW_ERR_UNSUPPORTED;
     return HW_OK;
 }
 
@@ -76,10 +77,12 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     // further row groups that read the same KV; more: 128-row workgroups whose waves share every K/V tile through
     // LDS (16-bit types, lengths known on the host) -- a CU can take in about 16 B/clk, so what counts is that every
     // CU reads every byte once
-    const bool wide_ok = p->dtype != HW_F32 && p->len_dev == nullptr && p->variant == HW_VARIANT_MFMA;
+    const bool wide_ok = p->dtype != HW_F32 && p->len_dev == nullptr && p->variant == HW_VARIANT_MFMA && p->E <= 128;
     plan->row_blocks = rows <= 16 ? 1 : 2;
     if (wide_ok && rows > 96) plan->row_blocks = hw::WIDE_ROW_BLOCKS;   // measured crossover: 95 rows 19.2 (narrow) / 19.9 us, 120 rows 21.8 / 20.6 us
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
+    // head dimension 256: kernels with one 16-row block only (two blocks of 256-wide accumulators do not fit the registers)
+    if (p->E > 128) plan->row_blocks = 1;
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rows_per_wg = 16 * plan->row_blocks;
     plan->row_groups = (rows + rows_per_wg - 1) / rows_per_wg;
@@ -99,7 +102,7 @@ int make_plan(const hw_problem* p, int num_cus, hw_plan* plan, int fused) {
     int wgs = p->splits;
     if (wgs <= 0) {
         // the two-row-block and fp32 kernels are built for one wave per SIMD (one workgroup per CU)
-        const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32) ? 2 : 1;
+        const int per_cu = (plan->row_blocks == 1 && p->dtype != HW_F32 && p->E <= 128) ? 2 : 1;
         const int target = per_cu * num_cus;
         wgs = target / (p->Hkv * plan->row_groups);
         // narrow kernels deal a workgroup's tiles to its four waves; in the wide kernel the whole workgroup takes every tile
@@ -230,7 +233,8 @@ int paged_validate(const hw_paged_problem* p) {
     }
     if (p->key_cache == nullptr || p->value_cache == nullptr || p->block_table == nullptr) return HW_ERR_NULL;
     if (!aligned16(p->out) || !aligned16(p->q) || !aligned16(p->key_cache) || !aligned16(p->value_cache)) return HW_ERR_ALIGN;
-    if (p->E != p->Ev || (p->E != 64 && p->E != 128)) return HW_ERR_UNSUPPORTED;
+    if (p->E != p->Ev || (p->E != 64 && p->E != 128 && p->E != 256)) return HW_ERR_UNSUPPORTED;
+    if (p->E == 256 && p->dtype == HW_F32) return HW_ERR_UNSUPPORTED;   // the paged kernel's two fp32 K tiles per wave exceed the LDS
     return HW_OK;
 }
 
@@ -258,10 +262,10 @@ int paged_plan(const hw_paged_problem* p, int num_cus, hw_paged_plan* plan) {
     // four sequences of 12 528 tokens with 3 / 6 / 12 / 19 query tokens each (15 ... 95 rows per sequence): 36.7 / 36.7 /
     // 45.9 / 69.4 us against 49.4 / 49.5 / 84.6 / 84.7 us of the 32-row workgroups, which stream a sequence's KV once per
     // 32 rows; with one token each (5 rows) the two are equal (36.0 / 36.1 us).
-    const bool wide_ok = p->dtype != HW_F32 && p->max_blocks <= hw::PAGED_WIDE_MAX_BLOCKS;
+    const bool wide_ok = p->dtype != HW_F32 && p->max_blocks <= hw::PAGED_WIDE_MAX_BLOCKS && p->E <= 128;
     if (wide_ok && rows_per_worker > 16) plan->row_blocks = hw::WIDE_ROW_BLOCKS;
     if (p->row_blocks == 1 || p->row_blocks == 2 || (p->row_blocks == hw::WIDE_ROW_BLOCKS && wide_ok)) plan->row_blocks = p->row_blocks;
-    if (p->dtype == HW_F32) plan->row_blocks = 1;   // the fp32 paged kernel exists with one row block only
+    if (p->dtype == HW_F32 || p->E > 128) plan->row_blocks = 1;   // the fp32 and the 256-wide paged kernels exist with one row block only
     const bool wide = plan->row_blocks == hw::WIDE_ROW_BLOCKS;
     const int rpw = 16 * plan->row_blocks;
     long long items;

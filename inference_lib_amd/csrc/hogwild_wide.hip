@@ -1148,6 +1148,7 @@ static hipError_t launch_wide_dt(const KernelArgs& ka, int E, hipStream_t stream
     constexpr int NS = WIDE_SLOTS;
     constexpr int NW = WIDE_WAVES;
     constexpr int PAR = WIDE_PAR;
+    if (E != 64 && E != 128) return hipErrorInvalidValue;
     if (ka.h.flags & KH_PREROTATED) {
         if (E == 128) hipLaunchKernelGGL((attention_wide_kernel<DT, 128, 128, NS, true, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
         else hipLaunchKernelGGL((attention_wide_kernel<DT, 64, 64, NS, true, NW, PAR>), dim3(ka.h.nwg), dim3(NW * 64), 0, stream, ka);
@@ -1186,6 +1187,7 @@ static hipError_t launch_paged_wide_dt(const PagedHeader& ph, int E, hipStream_t
     constexpr int NS = PAGED_WIDE_SLOTS;
     constexpr int NW = PAGED_WIDE_WAVES;
     constexpr int PAR = PAGED_WIDE_PAR;
+    if (E != 64 && E != 128) return hipErrorInvalidValue;
     if (E == 128) hipLaunchKernelGGL((paged_wide_kernel<DT, 128, 128, NS, NW, PAR>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
     else hipLaunchKernelGGL((paged_wide_kernel<DT, 64, 64, NS, NW, PAR>), dim3(ph.nwg), dim3(NW * 64), 0, stream, ph);
     return hipGetLastError();

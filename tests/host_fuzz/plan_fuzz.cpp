@@ -43,11 +43,12 @@ static void fuzz_fragments(std::mt19937_64& rng) {
     p.Hq = p.Hkv * (int)(U(0, 9) == 0 ? U(1, 4095) : U(1, 16));
     p.W = (int)(U(0, 9) == 0 ? U(1, 5000) : U(1, 16));
     p.S = (int)(U(0, 9) == 0 ? U(1, 4095) : U(1, 8));
-    p.E = p.Ev = U(0, 1) ? 128 : 64;
+    const int dims[3] = {64, 128, 256};
+    p.E = p.Ev = dims[U(0, 2)];
     p.RotE = p.E;
     p.scale = 0.1f;
     p.splits = U(0, 3) == 0 ? (int)U(1, 300) : 0;
-    p.row_blocks = (int)U(0, 2);
+    p.row_blocks = (int)(U(0, 6) == 0 ? 8 : U(0, 2));
     std::vector<int32_t> len(p.F);
     for (auto& l : len) {
         switch (U(0, 5)) {
@@ -74,6 +75,8 @@ static void fuzz_fragments(std::mt19937_64& rng) {
     const int rows = p.W * p.S * (p.Hq / p.Hkv);
     CHECK(plan.rows == rows && plan.tiles_per_head == tiles, "rows / tiles");
     CHECK(plan.row_blocks == 1 || plan.row_blocks == 2 || plan.row_blocks == 8, "row_blocks %d", plan.row_blocks);
+    if (p.E == 256) CHECK(plan.row_blocks == 1, "head dimension 256 planned with %d row blocks", plan.row_blocks);
+    if (p.dtype == HW_F32) CHECK(plan.row_blocks != 8, "fp32 planned with 128-row workgroups");
     CHECK((long long)plan.row_groups * 16 * plan.row_blocks >= rows && (long long)(plan.row_groups - 1) * 16 * plan.row_blocks < rows, "row groups");
     const int wgs = plan.wgs_per_head;
     CHECK(wgs >= 1 && wgs <= HW_MAX_SPLITS, "wgs %d", wgs);
@@ -159,7 +162,7 @@ static void fuzz_paged(std::mt19937_64& rng) {
     p.F = (int)U(1, 8);
     p.Hkv = 1 << U(0, 3);
     p.Hq = p.Hkv * (int)U(1, 16);
-    p.E = p.Ev = 128;
+    p.E = p.Ev = U(0, 2) == 0 ? 256 : 128;
     p.W = (int)(U(0, 3) == 0 ? U(1, 100000) : U(1, 64));
     p.S = (int)U(1, 8);
     p.block_size = (int)(U(0, 3) == 0 ? U(1, 4095) : (1 << U(0, 7)));
@@ -190,6 +193,7 @@ static void fuzz_paged(std::mt19937_64& rng) {
     CHECK(plan.rows == tokens * gq, "rows");
     CHECK(plan.splits >= 1 && plan.splits <= 64, "splits %d", plan.splits);
     CHECK(plan.row_groups >= 1, "row groups");
+    if (p.E == 256) CHECK(plan.row_blocks == 1 && !plan.device_planned, "head dimension 256 planned with %d row blocks", plan.row_blocks);
     CHECK((long long)plan.workgroups == (long long)p.Hkv * plan.row_groups * plan.splits && plan.workgroups < (1 << 20), "workgroups");
     size_t need = (size_t)p.Hkv * plan.splits * (size_t)(plan.rows > 0 ? plan.rows : 1) * ((size_t)p.Ev + 2) * sizeof(float);
     if (plan.device_planned) {

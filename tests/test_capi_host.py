@@ -102,6 +102,9 @@ def test_validation_happens_on_the_host():
     assert v(_problem(L, scale=-1.0)) == -3
     assert v(_problem(L, E=96, Ev=96, RotE=96)) == -4       # valid but not instantiated: a hard error, never silent
     assert v(_problem(L, Ev=64)) == -4
+    assert v(_problem(L, E=256, Ev=256, RotE=256)) == 0     # head dimension 256: the kernels with one 16-row block
+    assert v(_problem(L, E=256, Ev=256, RotE=256, variant=1)) == -4
+    assert v(_problem(L, E=512, Ev=512, RotE=512)) == -4
     assert v(_problem(L, F=65)) == 0                        # beyond one launch's 64 fragments: several launches
     assert v(_problem(L, F=512)) == 0 and v(_problem(L, F=513)) == -5
     assert v(_problem(L, F=65, len_dev=0x1000)) == -4       # device-resident lengths: one launch only
@@ -375,3 +378,21 @@ def test_build_inputs_and_append_validate_on_the_host():
     assert app(len=13, n_new=4) == -3                                   # 13 + 4 rows do not fit a capacity of 16
     assert app(dst=None) == -1
     assert app(n_new=0) == 0                                            # nothing to append: success without a device
+
+
+def test_head_dim_256_plans_with_one_row_block():
+    """Head dimension 256 exists with one 16-row block per workgroup only: more rows become row groups of 16, one workgroup
+    per CU, and a request for two blocks or for the 128-row kernel is not honoured."""
+    L = _lib()
+    lens = [4096] + [2048] * 4
+    for rb in (0, 2, 8):
+        pl = L.plan(lens, W=4, S=1, Hq=40, Hkv=8, Ev=256, num_cus=256, row_blocks=rb)
+        assert pl.row_blocks == 1 and pl.row_groups == 2 and pl.workgroups <= 256
+        assert pl.workgroups == 8 * 2 * pl.wgs_per_head
+    pl = L.plan(lens, W=8, S=4, Hq=64, Hkv=8, Ev=256, num_cus=256)         # 256 rows per kv head
+    assert pl.row_blocks == 1 and pl.row_groups == 16
+    for rb in (0, 2, 8):
+        pp = L.paged_plan(W=2, Hq=40, Hkv=8, Ev=256, block_size=16, max_blocks=64, num_cus=256, S=12, row_blocks=rb)
+        assert pp.row_blocks == 1 and pp.row_groups == 2 * ((12 * 5 + 15) // 16)
+    pp = L.paged_plan(W=3, Hq=40, Hkv=8, Ev=256, block_size=16, max_blocks=64, num_cus=256, total_q=100)
+    assert pp.row_blocks == 1 and pp.device_planned == 0

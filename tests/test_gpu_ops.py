@@ -22,9 +22,10 @@ def test_torch_ops_are_the_hip_path():
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f16", "f32"])
-def test_wrappers_match_oracle(oracle, dtype):
+@pytest.mark.parametrize("E", [128, 256])
+def test_wrappers_match_oracle(oracle, dtype, E):
     from inference_lib_amd import attention, cases
-    c = cases.small_case(dtype=dtype, W=2, S=1, Hq=8, Hkv=2, E=128, lens=(300, 70, 129, 5, 9), seed=3, with_cur=True)
+    c = cases.small_case(dtype=dtype, W=2, S=1, Hq=8, Hkv=2, E=E, lens=(300, 70, 129, 5, 9), seed=3, with_cur=True)
     cd = c.to(_dev())
     print(f"case {c.name}", flush=True)
     W, Hq, S, E = cd.q.shape
