@@ -260,6 +260,20 @@ __device__ __forceinline__ void load_tile(TileRegs<DT, E, EV>& t, const FragView
     }
 }
 
+// The wait in front of a tile's operand reads, stated by hand: the K transfers of the tile about to be multiplied have
+// landed when at most the operations issued behind them are outstanding -- the tile's own V loads and everything of the
+// AHEAD tiles requested after it (loads and transfers complete in issue order, and a tile is the same number of
+// instructions whether or not it exists).  The compiler places this wait itself from its own count of the operations in
+// flight, which ends at 63: with the 32 transfers + 32 loads of a 256-wide fp32 tile it placed none, and the operand reads
+// raced with the transfers.  So the kernels state it wherever a tile and its look-ahead come to 64 operations or more
+// (head dimension 256); where the compiler's own wait is present as well, the two agree.
+template <class G, int AHEAD>
+__device__ __forceinline__ void wait_k_landed() {
+    constexpr int BEHIND = 8 * G::NVL + AHEAD * (G::KL + 8 * G::NVL);
+    static_assert(BEHIND <= 63, "beyond the counter's range");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(BEHIND) : "memory");
+}
+
 // V image for transposed reads (the kernels whose waves share every tile, 16-bit types): rows of VROW bytes, the 32-byte
 // segments of a row (16 elements: what one MFMA block of outputs needs) stored at segment ^ key(row), the key chosen so
 // that the eight consecutive rows two neighbouring 16-lane groups read (2 x 4 rows x 32 bytes) cover all 64 banks:

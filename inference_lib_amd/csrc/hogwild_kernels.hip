@@ -257,6 +257,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
                 const int nb = (i + PF - 1) % PF;   // constant after unrolling
                 const int ln = l + (PF - 1) * NWAVES;
                 load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
+                if constexpr (E > 128) wait_k_landed<G, PF - 1>();
                 compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, l * TILE, n, q, a.sc, kslots[i]);
             }
         }
@@ -268,6 +269,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void attention_kernel(const KernelA
                 const int nb = (i + PF - 1) % PF;
                 const int ln = l + (PF - 1) * NWAVES;
                 load_tile<DT, E, EV>(tr[nb], fv, kslots[nb], koff, ln * TILE, n, q, ln < lt1);
+                if constexpr (E > 128) wait_k_landed<G, PF - 1>();
                 const bool live = l < lt1 && t0 < maxlim;
                 if (G::SZ == 4 && live && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);
                 else if (live) compute_tile<DT, E, EV, RB, true, QREG, VS>(tr[i], q_lds, qreg, lim, st, t0, n, q, a.sc, kslots[i]);

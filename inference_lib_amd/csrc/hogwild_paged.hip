@@ -212,12 +212,14 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
                 {
                     const int bt_n = bt_load(t + 2 * NW);
                     issue_tile(tr[1], kslots[1], bt_b, t + NW);
+                    if constexpr (E > 128) wait_k_landed<G, 1>();   // (see wait_k_landed: the table load in between only adds to what is behind)
                     compute_tile<DT, E, EV, RB, false, QREG>(tr[0], q_lds, qreg, lim, st, t * TILE, n, q, ph.sc, kslots[0]);
                     bt_a = bt_n;
                 }
                 {
                     const int bt_n = bt_load(t + 3 * NW);
                     issue_tile(tr[0], kslots[0], bt_a, t + 2 * NW);
+                    if constexpr (E > 128) wait_k_landed<G, 1>();
                     compute_tile<DT, E, EV, RB, false, QREG>(tr[1], q_lds, qreg, lim, st, (t + NW) * TILE, n, q, ph.sc, kslots[1]);
                     bt_b = bt_n;
                 }
@@ -226,6 +228,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
                 {
                     const int bt_n = bt_load(t + 2 * NW);
                     issue_tile(tr[1], kslots[1], bt_b, t + NW);
+                    if constexpr (E > 128) wait_k_landed<G, 1>();
                     const int t0 = t * TILE;
                     if (G::SZ == 4 && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
                     else compute_tile<DT, E, EV, RB, true, QREG>(tr[0], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[0]);
@@ -234,6 +237,7 @@ __global__ __launch_bounds__(NTHREADS, MINW) void paged_attention_kernel(const P
                 {
                     const int bt_n = bt_load(t + 3 * NW);
                     issue_tile(tr[0], kslots[0], bt_a, t + 2 * NW);
+                    if constexpr (E > 128) wait_k_landed<G, 1>();
                     const int t0 = (t + NW) * TILE;
                     if (G::SZ == 4 && t0 + TILE <= minlim) compute_tile<DT, E, EV, RB, false, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);
                     else if (t0 < maxlim) compute_tile<DT, E, EV, RB, true, QREG>(tr[1], q_lds, qreg, lim, st, t0, n, q, ph.sc, kslots[1]);

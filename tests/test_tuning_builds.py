@@ -93,3 +93,45 @@ def test_tile_loops_of_the_128_row_kernels_wait_only_for_their_own_transfers(tmp
                 elif not in_asm:
                     m = re.search(r"s_waitcnt[^\n]*vmcnt\((\d+)\)", line)
                     assert not (m and issued and int(m.group(1)) < issued), f"{name} {label}: {line.strip()} behind {issued} transfers"
+
+
+def test_one_buffer_kernels_wait_for_the_transfers_of_the_tile_they_multiply(tmp_path):
+    """The fp32 kernels keep one K tile per wave in LDS: a tile is requested (global->LDS transfers, then the V loads into
+    registers) and multiplied right away, so between a tile's last transfer and the first operand read out of LDS there
+    has to be a wait that leaves at most the loads issued behind the transfers in flight.  The compiler derives that wait
+    from its own count of the operations in flight and stopped placing it when a tile became 64 of them (256-wide fp32
+    rows: 32 transfers + 32 loads); the kernel states it itself there.  Checked in the generated code of every
+    one-buffer instantiation."""
+    if shutil.which(HIPCC) is None and not os.path.exists(HIPCC):
+        pytest.skip("no hipcc")
+    import re
+    from inference_lib_amd import build
+    asm = tmp_path / "kernels.s"
+    cmd = [HIPCC, f"--offload-arch={build.ARCH}", "-O3", "-std=c++17", "-fno-gpu-rdc", "-munsafe-fp-atomics", "--cuda-device-only",
+           *build.DEVICE_FLAGS, "-I", os.path.join(ROOT, "include"), "-S", os.path.join(build.CSRC, "hogwild_kernels.hip"), "-o", str(asm)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, r.stderr[-3000:]
+    text = asm.read_text()
+    # attention_kernel<DT, E, EV, RB, MINW, PF, ...>: PF == 1 is the one-buffer form
+    kernels = re.findall(r"^(_ZN2hw16attention_kernelINS_\w+?ELi\d+ELi\d+ELi\d+ELi\d+ELi1ELb\S*):", text, re.M)
+    assert len(kernels) >= 12 and any("ELi256ELi256" in k for k in kernels), kernels
+    groups = 0
+    for name in kernels:
+        body = text[text.index(name + ":"):]
+        body = body[:body.index("; -- End function")]
+        pending, younger = False, 0
+        for line in body.splitlines():
+            t = line.strip()
+            if re.match(r"buffer_load_dwordx4 .*\blds\b", t):
+                if not pending:
+                    groups += 1
+                pending, younger = True, 0
+            elif re.match(r"(global|buffer)_load_", t):
+                younger += 1
+            elif t.startswith("s_waitcnt"):
+                m = re.search(r"vmcnt\((\d+)\)", t)
+                if m and int(m.group(1)) <= younger:
+                    pending = False
+            elif t.startswith("ds_read"):
+                assert not pending, f"{name}: {t} with the tile's transfers possibly in flight ({younger} loads behind them)"
+    assert groups >= len(kernels)
