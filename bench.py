@@ -46,7 +46,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--case", type=int, default=3, help="workload configuration 1..5 (3 = headline)")
+    ap.add_argument("--case", type=int, default=3, help="workload configuration 1..5 (3 = headline); 6 = the headline's fragments at head dimension 256")
     ap.add_argument("--splits", type=int, default=0, help="workgroups per kv head (0 = library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg (and with it the parity gate)")
     ap.add_argument("--no-rq", action="store_true", help="do not write the rotated-query side output")
@@ -306,7 +306,7 @@ def side_config(case_id, dev, args, stream):
            "step_us_p10_p90": [round(step["p10"], 3), round(step["p90"], 3)],
            "kernel_frac_of_peak": round(run.kv_bytes / kern["median"] / 1e3 / PEAK_HBM_GBS, 4),
            "step_GBps": round(run.kv_bytes / step["median"] / 1e3, 1)}
-    if run.plan.rows <= 16 and args.variant == "mfma":
+    if run.plan.rows <= 16 and args.variant == "mfma" and run.case.E <= 128:
         # the matrix-core choice measured against VALU logits on the same workload (same ring, same plan)
         del run
         torch.cuda.empty_cache()
@@ -539,7 +539,7 @@ def main():
         del run, problems, problems_dl
         torch.cuda.empty_cache()
         cfgs = []
-        for cid in (1, 2, 4, 5):
+        for cid in (1, 2, 4, 5, 6):
             if cid != args.case:
                 cfgs.append(side_config(cid, dev, args, stream))
         for wl in ("paged", "varlen"):

@@ -118,7 +118,7 @@ def _prompt_segments_orders(W: int, with_cur: bool) -> List[List[int]]:
 
 
 def baseline_case(idx: int) -> Case:
-    """The five workload configurations, numbered 1..5 (config 3 is the benchmark headline)."""
+    """The five workload configurations, numbered 1..5 (config 3 is the benchmark headline), and 6: head dimension 256."""
     g = torch.Generator().manual_seed(idx - 1)
     if idx == 1:   # fp32 parity case: prompt 256 + one 64-token segment per worker, fragment order
         # = worker 0's ordering [prompt, seg1, seg0]
@@ -139,6 +139,11 @@ def baseline_case(idx: int) -> Case:
     if idx == 5:   # multi-token step, fp16
         lens = [8192] + [2048] * 4
         return build_case("c5_multitoken_w4s4", "f16", 4, 4, 64, 8, 128, 1e6, lens, _prompt_segments_orders(4, False), g)
+    if idx == 6:   # not one of the reference's configurations: the headline's fragments at head dimension 256
+        # (the Gemma-2-9B head shape: 16 query heads on 8 kv heads), 4 workers
+        cur = torch.randint(1, 129, (4,), generator=g).tolist()
+        lens = [4096] + [2048] * 4 + cur
+        return build_case("c6_gemma9b_w4_d256", "bf16", 4, 1, 16, 8, 256, 1e4, lens, _prompt_segments_orders(4, True), g)
     raise ValueError(f"no such baseline case: {idx}")
 
 

@@ -28,7 +28,7 @@ def test_small_fused(oracle, dtype, E):
     assert_close("lse", lse, l_ref, TOL[dtype])
 
 
-@pytest.mark.parametrize("idx", [1, 2, 3, 4, 5])
+@pytest.mark.parametrize("idx", [1, 2, 3, 4, 5, 6])
 def test_baseline_configs(oracle, idx):
     from inference_lib_amd import cases
     c = cases.baseline_case(idx)
