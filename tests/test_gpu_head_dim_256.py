@@ -138,3 +138,57 @@ def test_what_head_dim_256_does_not_have():
         _lib.Problem(q=cs.q, locations=cs.locations, keys=cs.keys, values=cs.values, scale=cs.scale, out=o, cosines=cs.cos,
                      sines=cs.sin, variant=_lib.HW_VARIANT_VALU_QK).run()
     assert ei.value.status == -4     # HW_ERR_UNSUPPORTED
+
+
+EDGE = [0, 1, 2, 15, 16, 17, 31, 32, 33, 63, 64, 65, 95, 96, 97, 127, 128, 129, 255, 256, 257, 1000, 1023, 1025]
+
+
+@pytest.mark.parametrize("seed", range(18))
+def test_fused_random_shapes_head_dim_256(oracle, seed):
+    """Random shapes as in test_gpu_random.py, at head dimension 256: fragment lengths around the tile size, empty fragments,
+    random worker orders, 1..9 workers, several query tokens, GQA 1..7 and 16, explicit split factors, all three dtypes."""
+    from inference_lib_amd import cases
+    rng = np.random.default_rng(25600 + seed)
+    dtype = ["bf16", "f16", "f32"][seed % 3]
+    W = int(rng.integers(1, 10))
+    S = int(rng.choice([1, 1, 1, 2, 3]))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    GQ = 16 if seed % 9 == 8 else int(rng.integers(1, 8))
+    F = int(rng.integers(1, 13))
+    lens = [int(rng.choice(EDGE)) if rng.random() < 0.7 else int(rng.integers(0, 3000)) for _ in range(F)]
+    if sum(lens) == 0:
+        lens[0] = 40
+    orders = [[int(x) for x in rng.permutation(F)] for _ in range(W)]
+    c = cases.build_case(f"rand256_{seed}", dtype, W, S, Hkv * GQ, Hkv, 256, 1e4, lens, orders, torch.Generator().manual_seed(seed))
+    splits = int(rng.choice([0, 0, 1, 3, 7, 40]))
+    print(f"seed {seed}: {dtype} W={W} S={S} Hq={Hkv * GQ} Hkv={Hkv} lens={lens} splits={splits}", flush=True)
+    want_o, want_l, want_rq = oracle_fused(oracle, c)
+    out, lse, rq = run_fused(c.to(_dev()), splits=splits)
+    assert_close("out", out, want_o, TOL[dtype])
+    assert_close("lse", lse, want_l, TOL[dtype])
+    assert_close("rq", rq, want_rq, 1e-5 if dtype == "f32" else 3.2e-2)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_paged_random_shapes_head_dim_256(seed):
+    rng = np.random.default_rng(25700 + seed)
+    dtype = ["bf16", "f16"][seed % 2]
+    W = int(rng.integers(1, 7))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    GQ = int(rng.integers(1, 8))
+    bs = int(rng.choice([1, 4, 8, 16, 16, 32, 48, 64, 256]))
+    F = int(rng.integers(1, 4))
+    varlen = bool(rng.random() < 0.4)
+    S = int(rng.choice([1, 1, 2, 5]))
+    longest = int(rng.choice([40, 130, 700, 2100]))
+    seq = [int(rng.integers(S + 3 * F + 1, longest + S + 3 * F + 2)) for _ in range(W)]
+    mb = (max(seq) + bs - 1) // bs + int(rng.integers(0, 3))
+    kw = dict(seed=seed, loc_mode="random" if rng.random() < 0.5 else "causal")
+    if varlen:
+        ql = [int(min(s - 3 * F, x)) for s, x in zip(seq, rng.integers(0, 7, size=W))]
+        if sum(ql) == 0:
+            ql[0] = 1
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, 256, bs, mb, seq_lens=seq, q_lens=ql, **kw)
+    else:
+        c = build_paged(dtype, F, W, Hkv * GQ, Hkv, 256, bs, mb, seq_lens=seq, S=S, **kw)
+    check_paged(c, splits=int(rng.choice([0, 0, 1, 5])))
