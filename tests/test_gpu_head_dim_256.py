@@ -192,3 +192,23 @@ def test_paged_random_shapes_head_dim_256(seed):
     else:
         c = build_paged(dtype, F, W, Hkv * GQ, Hkv, 256, bs, mb, seq_lens=seq, S=S, **kw)
     check_paged(c, splits=int(rng.choice([0, 0, 1, 5])))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_repeated_runs_are_bit_identical_head_dim_256(dtype):
+    """The same call repeated with the caches overwritten in between gives the same bits every time.  (A 256-wide fp32
+    tile is 64 vector-memory operations in flight; the operand reads once ran ahead of the tile's transfers and the result
+    depended on how fast memory answered.)"""
+    from inference_lib_amd import cases
+    c = cases.small_case(dtype=dtype, W=4, S=2, Hq=8, Hkv=2, E=256, lens=(900, 40, 33, 64, 1), seed=21)
+    cd = c.to(_dev())
+    flush = torch.empty(384 * 1024 * 1024, dtype=torch.uint8, device=_dev())
+    ref = None
+    for rep in range(25):
+        flush.fill_(rep)
+        out, lse, rq = run_fused(cd)
+        cur = [t.clone().view(torch.uint8) for t in (out, lse, rq)]
+        if ref is None:
+            ref = cur
+        else:
+            assert all(torch.equal(a, b) for a, b in zip(ref, cur)), f"run {rep} differs from the first"
