@@ -522,13 +522,13 @@ static hipError_t launch_merge_ev(const MergeArgs& ma, hipStream_t stream) {
         const int blocks = ma.Hkv * ((ma.R + RPW - 1) / RPW);
         hipLaunchKernelGGL((merge_kernel<DT, EV, RPW>), dim3(blocks), dim3(256), 0, stream, ma);
     };
-    bool eight = false;
-    if constexpr (NPG >= 8) {
-        eight = ns <= 4;
-        if (eight) go(std::integral_constant<int, 8>{});
+    if constexpr (NPG >= 8) {       // (eight rows side by side need eight thread groups: not at head dimension 256)
+        if (ns <= 4) {
+            go(std::integral_constant<int, 8>{});
+            return hipGetLastError();
+        }
     }
-    if (eight) {}
-    else if (ns <= 4 * (NPG / 4)) go(std::integral_constant<int, 4>{});
+    if (ns <= 4 * (NPG / 4)) go(std::integral_constant<int, 4>{});
     else if (ns <= 4 * (NPG / 2)) go(std::integral_constant<int, 2>{});
     else go(std::integral_constant<int, 1>{});
     return hipGetLastError();
